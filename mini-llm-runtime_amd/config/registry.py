@@ -34,8 +34,10 @@ def config_class(name):
 
 def config_from_dict(data):
     archs = data.get("architectures")
+    if archs is None and isinstance(data.get("architecture"), str):      # (one name under the singular key)
+        archs = [data["architecture"]]
     if not isinstance(archs, list) or len(archs) != 1 or not isinstance(archs[0], str):
-        raise ConfigError("config.json needs `architectures` with exactly one name")
+        raise ConfigError("config.json needs `architectures` with exactly one name (or `architecture`, a name)")
     return config_class(archs[0]).from_dict(data)
 
 

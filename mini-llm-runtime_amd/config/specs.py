@@ -48,11 +48,77 @@ class MlpSpec:
 
 
 @dataclass(frozen=True)
+class QueryTemperature:
+    """A factor on the query that grows with its position p: 1 + coef * ln(floor((p + 1) / every) + 1)."""
+    coef: float
+    every: float
+
+
+@dataclass(frozen=True)
+class DiffAttentionSpec:
+    """Differential attention: every query head holds two maps (two softmax attentions over the same
+    values); the head's output is map 1 - lam * map 2, divided by its root mean square and scaled by
+    `out_scale`, then gated."""
+    kind: str                 # "diff_attention"
+    hidden: int
+    q_heads: int
+    kv_heads: int
+    head_dim: int             # query/key channels of ONE map
+    value_dim: int
+    scale: float
+    lam_init: float           # the constant in lam = exp(lq1 . lk1) - exp(lq2 . lk2) + lam_init
+    out_scale: float          # factor on the normed difference
+    eps: float
+    softcap: Optional[float] = None           # score <- softcap * tanh(score / softcap)
+    q_temperature: Optional[QueryTemperature] = None
+    gate: Optional[str] = "sigmoid"           # activation of the output gate (None: no gate)
+
+
+@dataclass(frozen=True)
+class GlaSpec:
+    """Gated linear attention: per head S_t = diag(alpha_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, the decay
+    alpha_t = sigmoid(z_t)^(1 / tau) per key channel from a low-rank pair of projections."""
+    kind: str                 # "gla"
+    hidden: int
+    heads: int
+    head_dim: int
+    value_dim: int
+    decay_rank: int
+    tau: float
+    eps: float
+
+
+@dataclass(frozen=True)
+class Mamba2Spec:
+    """Mamba-2 (state-space duality): a short causal convolution over x, B, C, then per head
+    S_t = exp(-exp(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T, y_t = S_t^T C_t + D x_t, gated and normed in groups."""
+    kind: str                 # "mamba2"
+    hidden: int
+    heads: int
+    value_dim: int
+    state: int
+    groups: int
+    conv_taps: int
+    norm_groups: int
+    eps: float
+
+
+@dataclass(frozen=True)
+class ClampedGluSpec:
+    """g = min(gate, limit), u = clamp(up, -limit, limit), y = g * sigmoid(slope * g) * (u + 1)."""
+    kind: str                 # "clamped_glu"
+    hidden: int
+    intermediate: int
+    limit: float
+    slope: float = 1.702
+
+
+@dataclass(frozen=True)
 class LayerSpec:
-    kind: str                 # key in the block registry, e.g. "prenorm"
+    kind: str                 # key in the block registry, e.g. "prenorm", "parallel"
     norm1: NormSpec
     mixer: object             # any mixer spec with a `kind`
-    norm2: NormSpec
+    norm2: Optional[NormSpec]     # None with `ffn` None: a layer without a feed-forward
     ffn: object               # any feed-forward spec with a `kind`
 
 

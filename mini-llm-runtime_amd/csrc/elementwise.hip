@@ -323,6 +323,99 @@ __global__ void finite_check_kernel(const float* __restrict__ h, const elem_t* _
     }
 }
 
+
+// A layer whose mixer and feed-forward read the SAME input through norms of their own: x = h + d1 + d2 (what
+// the layer before still has to add; either may be null), written back to h; out1 = (x * r) * w1 and
+// out2 = (x * r) * w2 with the one r = rsqrt(mean(x^2) + eps) that both norms share (out2 / w2 may be null).
+// One workgroup per row, the sum of squares in a fixed order.
+__global__ void add2_rmsnorm2_kernel(float* __restrict__ h, const elem_t* __restrict__ d1, const elem_t* __restrict__ d2,
+                                     const float* __restrict__ w1, const float* __restrict__ w2,
+                                     elem_t* __restrict__ out1, elem_t* __restrict__ out2, int width, float eps) {
+    __shared__ float scratch[16];
+    const size_t r = blockIdx.x;
+    float* hrow = h + r * width;
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float x = hrow[i];
+        if (d1 || d2) {
+            float add = d1 ? to_float(d1[r * width + i]) : 0.f;
+            if (d2) add += to_float(d2[r * width + i]);
+            x += add;
+            hrow[i] = x;
+        }
+        sum += x * x;
+    }
+    sum = block_sum(sum, scratch);
+    const float scale = 1.0f / sqrtf(sum / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float x = hrow[i] * scale;           // (this thread wrote hrow[i] itself)
+        out1[r * width + i] = from_float<elem_t>(x * w1[i]);
+        if (out2) out2[r * width + i] = from_float<elem_t>(x * w2[i]);
+    }
+}
+
+// h += d1 + d2 (d2 may be null): the two branches of such a layer added in 32-bit when no norm follows.
+__global__ void residual_add2_kernel(float* __restrict__ h, const elem_t* __restrict__ d1, const elem_t* __restrict__ d2,
+                                     size_t count) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
+        float add = to_float(d1[i]);
+        if (d2) add += to_float(d2[i]);
+        h[i] += add;
+    }
+}
+
+// act[m, f] = g * sigmoid(slope * g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit);
+// gate = gate_up[m, f], up = gate_up[m, inter + f].
+__global__ void clamped_glu_kernel(const elem_t* __restrict__ gate_up, elem_t* __restrict__ act, int rows, int inter,
+                                   float limit, float slope) {
+    const size_t total = (size_t)rows * inter;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t m = i / inter, f = i % inter;
+        const float g = fminf(to_float(gate_up[m * 2 * inter + f]), limit);
+        const float u = fminf(fmaxf(to_float(gate_up[m * 2 * inter + inter + f]), -limit), limit);
+        act[i] = from_float<elem_t>((g / (1.0f + expf(-slope * g))) * (u + 1.0f));
+    }
+}
+
+// The end of a recurrent mixer: y [rows, width] float is cut into parts of `part` values, each divided by its
+// own root mean square (eps inside the root) and multiplied by weight[i % period]; the gate (an activation of
+// gate[m, i], read with a row stride of its own) multiplies before the norm (gate_first) or after it.
+// One wavefront per (row, part); gate_kind 0: silu, 1: sigmoid.
+__global__ __launch_bounds__(256) void gated_part_norm_kernel(const float* __restrict__ y, const elem_t* __restrict__ gate,
+                                                              long gate_stride, const float* __restrict__ weight,
+                                                              elem_t* __restrict__ out, int rows, int width, int part,
+                                                              int period, float eps, int gate_first, int gate_kind) {
+    const int lane = threadIdx.x & 63;
+    const size_t unit = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int parts = width / part;
+    if (unit >= (size_t)rows * parts) return;
+    const size_t m = unit / parts;
+    const int c0 = (int)(unit % parts) * part;
+    const float* yrow = y + m * width;
+    const elem_t* grow = gate + m * gate_stride;
+    auto gate_of = [&](int c) {
+        const float z = to_float(grow[c]);
+        const float s = 1.0f / (1.0f + expf(-z));
+        return gate_kind == 0 ? z * s : s;
+    };
+    float sum = 0.f;
+    for (int i = lane; i < part; i += 64) {
+        float v = yrow[c0 + i];
+        if (gate_first) v *= gate_of(c0 + i);
+        sum += v * v;
+    }
+    sum = wave_sum(sum);
+    const float scale = 1.0f / sqrtf(sum / (float)part + eps);
+    for (int i = lane; i < part; i += 64) {
+        const int c = c0 + i;
+        float v = yrow[c];
+        if (gate_first) v *= gate_of(c);
+        v = (v * scale) * weight[c % period];
+        if (!gate_first) v *= gate_of(c);
+        out[m * width + c] = from_float<elem_t>(v);
+    }
+}
+
 static int grid_for(size_t count, int block) {
     size_t g = (count + block - 1) / block;
     return (int)(g > 65535 ? 65535 : (g == 0 ? 1 : g));
@@ -391,6 +484,39 @@ int mlr_silu_mul(const void* gate_up, void* act, int rows, int inter, hipStream_
     }
     silu_mul_kernel<<<grid_for((size_t)rows * inter, 256), 256, 0, stream>>>(
         (const elem_t*)gate_up, (elem_t*)act, rows, inter);
+    return (int)hipGetLastError();
+}
+
+int mlr_add2_rmsnorm2(float* h, const void* d1, const void* d2, const float* w1, const float* w2, void* out1, void* out2,
+                      int rows, int width, float eps, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if ((out2 == nullptr) != (w2 == nullptr)) return -1;
+    add2_rmsnorm2_kernel<<<rows, 256, 0, stream>>>(h, (const elem_t*)d1, (const elem_t*)d2, w1, w2, (elem_t*)out1,
+                                                   (elem_t*)out2, width, eps);
+    return (int)hipGetLastError();
+}
+
+int mlr_residual_add2(float* h, const void* d1, const void* d2, size_t count, hipStream_t stream) {
+    if (count == 0) return 0;
+    residual_add2_kernel<<<grid_for(count, 256), 256, 0, stream>>>(h, (const elem_t*)d1, (const elem_t*)d2, count);
+    return (int)hipGetLastError();
+}
+
+int mlr_clamped_glu(const void* gate_up, void* act, int rows, int inter, float limit, float slope, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    clamped_glu_kernel<<<grid_for((size_t)rows * inter, 256), 256, 0, stream>>>((const elem_t*)gate_up, (elem_t*)act, rows,
+                                                                              inter, limit, slope);
+    return (int)hipGetLastError();
+}
+
+int mlr_gated_part_norm(const float* y, const void* gate, long gate_stride, const float* weight, void* out, int rows,
+                        int width, int part, int period, float eps, int gate_first, int gate_kind, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (part <= 0 || width % part != 0 || period <= 0) return -1;
+    const size_t units = (size_t)rows * (width / part);
+    gated_part_norm_kernel<<<(unsigned)((units + 3) / 4), 256, 0, stream>>>(y, (const elem_t*)gate, gate_stride, weight,
+                                                                           (elem_t*)out, rows, width, part, period, eps,
+                                                                           gate_first, gate_kind);
     return (int)hipGetLastError();
 }
 

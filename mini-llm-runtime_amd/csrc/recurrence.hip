@@ -1,0 +1,249 @@
+// Mixers with a state of fixed size per request: a short causal convolution over channels, the decays of
+// gated linear attention and of Mamba-2, and the linear recurrence both share,
+//     S_t = diag(a_t) S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t        (S: N key channels x V value channels),
+// run token by token in 32-bit from the state that earlier steps left.  A step brings any mix of prompt
+// portions and single tokens; a request's tokens are consecutive rows of the batch (`seg_first`, `seg_count`,
+// one entry a request of the step).  The live state of a request is read from `live + slot * stride`, the
+// state that the step leads to is written to `stage + slot * stride` (the engine makes it live when every
+// layer has run).  Every sum is taken in an order that depends on the token's own data only, so a token's
+// result does not depend on how its request was cut into steps or on what else the batch holds.
+#include "common.h"
+
+__device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+
+// ---- short causal convolution -----------------------------------------------------------------------
+// out[r, c] = act(b[c] + sum_j w[c, j] * in(r, taps - 1 - j)) with in(r, d) the channel's input d tokens before
+// row r: a row of this step when the request brought it, else the request's state, which holds its last
+// taps - 1 inputs, oldest first, as [taps - 1][C] floats (zeros at a sequence's start).  The last row of a
+// request in the step writes the state that follows.  One thread per (row, channel).
+struct ConvArgs {
+    const elem_t* x; long x_stride;
+    const float* w; const float* b;
+    elem_t* out; long out_stride;
+    const float* live; float* stage; long state_stride;
+    const int32_t* slots; const int32_t* positions;
+    int rows, channels, taps, silu, write_state;
+};
+
+#define CONV_MAX_TAPS 8
+
+__global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
+    const int r = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    const int slot = a.slots[r], pos = a.positions[r];
+    const int before = a.taps - 1;
+    int have = 0;                              // rows right before r that are this request's previous tokens
+    while (have < before && r - have - 1 >= 0 && a.slots[r - have - 1] == slot && a.positions[r - have - 1] == pos - have - 1) ++have;
+    const bool last = r + 1 >= a.rows || a.slots[r + 1] != slot || a.positions[r + 1] != pos + 1;
+    if (c >= a.channels) return;
+    float in[CONV_MAX_TAPS];                   // in[d]: the input d tokens back
+#pragma unroll
+    for (int d = 0; d < CONV_MAX_TAPS; ++d) {
+        if (d > before) { in[d] = 0.f; continue; }
+        if (d <= have) in[d] = to_float(a.x[(size_t)(r - d) * a.x_stride + c]);
+        else in[d] = a.live[(size_t)slot * a.state_stride + (size_t)(before - d + have) * a.channels + c];
+    }
+    float acc = a.b ? a.b[c] : 0.f;
+#pragma unroll
+    for (int d = CONV_MAX_TAPS - 1; d >= 0; --d) {         // oldest input first; tap j = taps - 1 - d
+        if (d <= before) acc += a.w[(size_t)c * a.taps + (before - d)] * in[d];
+    }
+    if (a.silu) acc = acc / (1.0f + expf(-acc));
+    a.out[(size_t)r * a.out_stride + c] = from_float<elem_t>(acc);
+    if (last && a.write_state) {
+#pragma unroll
+        for (int d = 0; d < CONV_MAX_TAPS - 1; ++d) {
+            if (d < before) a.stage[(size_t)slot * a.state_stride + (size_t)(before - 1 - d) * a.channels + c] = in[d];
+        }
+    }
+}
+
+// ---- decays ---------------------------------------------------------------------------------------------
+// Gated linear attention: the logarithm of alpha = sigmoid(z + b)^(1 / tau), that is -softplus(-(z + b)) / tau.
+__global__ void gla_log_decay_kernel(const elem_t* __restrict__ z, const float* __restrict__ bias, float* __restrict__ out,
+                                     size_t rows, int width, float inv_tau) {
+    const size_t total = rows * width;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const float x = to_float(z[i]) + (bias ? bias[i % width] : 0.f);
+        out[i] = -softplus_f(-x) * inv_tau;
+    }
+}
+
+// Mamba-2: the step size dt = softplus(raw + dt_bias[h]) (no clamp) and the log decay -exp(A_log[h]) * dt.
+__global__ void mamba_step_kernel(const elem_t* __restrict__ raw, long raw_stride, const float* __restrict__ dt_bias,
+                                  const float* __restrict__ a_log, float* __restrict__ dt, float* __restrict__ log_decay,
+                                  size_t rows, int heads) {
+    const size_t total = rows * heads;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / heads;
+        const int h = (int)(i % heads);
+        const float step = softplus_f(to_float(raw[r * raw_stride + h]) + dt_bias[h]);
+        dt[i] = step;
+        log_decay[i] = -expf(a_log[h]) * step;
+    }
+}
+
+// ---- the recurrence --------------------------------------------------------------------------------------
+struct ScanArgs {
+    const elem_t* q; long q_stride;            // q[r * q_stride + (head / heads_per_group) * N + i]
+    const elem_t* k; long k_stride;
+    const elem_t* v; long v_stride;            // v[r * v_stride + head * V + j]
+    const float* log_decay; long decay_stride; // per channel: [r * stride + head * N + i]; else [r * stride + head]
+    const float* v_scale; long v_scale_stride; // factor on v, [r * stride + head], or null
+    const float* skip;                         // out += skip[head] * v (unscaled), or null
+    float* out;                                // [rows, heads * V]
+    const float* live; float* stage; long state_stride;     // a request's S as [heads][N][V]
+    const int32_t* seg_first; const int32_t* seg_count; const int32_t* slots;
+    int heads, heads_per_group, N, V, decay_per_channel, write_state;
+    float q_scale;
+};
+
+#define SCAN_COLS 64
+#define SCAN_PARTS 4
+
+// One workgroup per (request of the step, head, 64 value channels): wavefront p holds rows [p NR, (p + 1) NR)
+// of S for its 64 columns in registers, a lane a column.  Tokens are staged TILE at a time through LDS
+// (decays exponentiated, q scaled, v scaled); after a tile the four partial sums of o are added in the order
+// of the parts.
+template <int NR, int TILE>
+__global__ __launch_bounds__(256) void linear_recurrence_kernel(ScanArgs a) {
+    constexpr int NPAD = NR * SCAN_PARTS;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    float* a_lds = lds;                                   // [TILE][NPAD]
+    float* k_lds = a_lds + TILE * NPAD;
+    float* q_lds = k_lds + TILE * NPAD;
+    float* v_lds = q_lds + TILE * NPAD;                   // [TILE][COLS]
+    float* o_lds = v_lds + TILE * SCAN_COLS;              // [PARTS][TILE][COLS]
+    const int seg = blockIdx.x, head = blockIdx.y, col0 = blockIdx.z * SCAN_COLS;
+    const int r0 = a.seg_first[seg], n = a.seg_count[seg];
+    const int slot = a.slots[r0];
+    const int j = threadIdx.x & 63, part = threadIdx.x >> 6;
+    const int col = col0 + j;
+    const int N = a.N, V = a.V;
+    const int qk_head = head / a.heads_per_group;
+    const size_t state_at = (size_t)slot * a.state_stride + (size_t)head * N * V;
+    float S[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        const int i = part * NR + r;
+        S[r] = (i < N && col < V) ? a.live[state_at + (size_t)i * V + col] : 0.f;
+    }
+    for (int t0 = 0; t0 < n; t0 += TILE) {
+        const int nt = min(TILE, n - t0);
+        __syncthreads();                                  // the tile before is read and written out
+        for (int idx = threadIdx.x; idx < nt * NPAD; idx += 256) {
+            const int t = idx / NPAD, i = idx % NPAD;
+            const size_t row = (size_t)(r0 + t0 + t);
+            float da = 0.f, dk = 0.f, dq = 0.f;
+            if (i < N) {
+                da = expf(a.log_decay[row * a.decay_stride + (a.decay_per_channel ? head * N + i : head)]);
+                dk = to_float(a.k[row * a.k_stride + qk_head * N + i]);
+                dq = to_float(a.q[row * a.q_stride + qk_head * N + i]) * a.q_scale;
+            }
+            a_lds[idx] = da; k_lds[idx] = dk; q_lds[idx] = dq;
+        }
+        for (int idx = threadIdx.x; idx < nt * SCAN_COLS; idx += 256) {
+            const int t = idx / SCAN_COLS, c = col0 + idx % SCAN_COLS;
+            const size_t row = (size_t)(r0 + t0 + t);
+            float x = 0.f;
+            if (c < V) {
+                x = to_float(a.v[row * a.v_stride + head * V + c]);
+                if (a.v_scale) x *= a.v_scale[row * a.v_scale_stride + head];
+            }
+            v_lds[idx] = x;
+        }
+        __syncthreads();
+        for (int t = 0; t < nt; ++t) {
+            const float x = v_lds[t * SCAN_COLS + j];
+            const float* at = a_lds + t * NPAD + part * NR;
+            const float* kt = k_lds + t * NPAD + part * NR;
+            const float* qt = q_lds + t * NPAD + part * NR;
+            float o = 0.f;
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                S[r] = at[r] * S[r] + kt[r] * x;
+                o += qt[r] * S[r];
+            }
+            o_lds[(part * TILE + t) * SCAN_COLS + j] = o;
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < nt * SCAN_COLS; idx += 256) {
+            const int t = idx / SCAN_COLS, c = col0 + idx % SCAN_COLS;
+            if (c >= V) continue;
+            const size_t row = (size_t)(r0 + t0 + t);
+            float o = o_lds[idx];
+#pragma unroll
+            for (int p = 1; p < SCAN_PARTS; ++p) o += o_lds[p * TILE * SCAN_COLS + idx];
+            if (a.skip) o += a.skip[head] * to_float(a.v[row * a.v_stride + head * V + c]);
+            a.out[row * ((size_t)a.heads * V) + head * V + c] = o;
+        }
+    }
+    if (a.write_state && col < V) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int i = part * NR + r;
+            if (i < N) a.stage[state_at + (size_t)i * V + col] = S[r];
+        }
+    }
+}
+
+template <int NR, int TILE>
+static int launch_scan(const ScanArgs& a, int segments, hipStream_t stream) {
+    const size_t lds = sizeof(float) * ((size_t)3 * TILE * NR * SCAN_PARTS + (size_t)TILE * SCAN_COLS * (1 + SCAN_PARTS));
+    dim3 grid(segments, a.heads, (a.V + SCAN_COLS - 1) / SCAN_COLS);
+    linear_recurrence_kernel<NR, TILE><<<grid, 256, lds, stream>>>(a);
+    return (int)hipGetLastError();
+}
+
+static int grid_for(size_t count, int block) {
+    size_t g = (count + block - 1) / block;
+    return (int)(g > 65535 ? 65535 : (g == 0 ? 1 : g));
+}
+
+extern "C" {
+
+int mlr_causal_conv(const void* x, long x_stride, const float* w, const float* b, void* out, long out_stride,
+                    const float* live, float* stage, long state_stride, const int32_t* slots, const int32_t* positions,
+                    int rows, int channels, int taps, int silu, int write_state, hipStream_t stream) {
+    if (rows <= 0 || channels <= 0) return 0;
+    if (taps < 1 || taps > CONV_MAX_TAPS) return -1;
+    ConvArgs a{(const elem_t*)x, x_stride, w, b, (elem_t*)out, out_stride, live, stage, state_stride, slots, positions,
+               rows, channels, taps, silu, write_state};
+    causal_conv_kernel<<<dim3(rows, (channels + 255) / 256), 256, 0, stream>>>(a);
+    return (int)hipGetLastError();
+}
+
+int mlr_gla_log_decay(const void* z, const float* bias, float* out, int rows, int width, float inv_tau, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    gla_log_decay_kernel<<<grid_for((size_t)rows * width, 256), 256, 0, stream>>>((const elem_t*)z, bias, out, (size_t)rows,
+                                                                                 width, inv_tau);
+    return (int)hipGetLastError();
+}
+
+int mlr_mamba_step(const void* raw, long raw_stride, const float* dt_bias, const float* a_log, float* dt, float* log_decay,
+                   int rows, int heads, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    mamba_step_kernel<<<grid_for((size_t)rows * heads, 256), 256, 0, stream>>>((const elem_t*)raw, raw_stride, dt_bias, a_log,
+                                                                              dt, log_decay, (size_t)rows, heads);
+    return (int)hipGetLastError();
+}
+
+int mlr_linear_recurrence(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
+                          const float* log_decay, long decay_stride, int decay_per_channel, const float* v_scale,
+                          long v_scale_stride, const float* skip, float q_scale, float* out, const float* live, float* stage,
+                          long state_stride, const int32_t* seg_first, const int32_t* seg_count, const int32_t* slots,
+                          int segments, int heads, int heads_per_group, int n_keys, int n_values, int write_state,
+                          hipStream_t stream) {
+    if (segments <= 0) return 0;
+    if (n_keys < 1 || n_keys > 256 || n_values < 1 || heads < 1 || heads_per_group < 1 || heads % heads_per_group) return -1;
+    ScanArgs a{(const elem_t*)q, q_stride, (const elem_t*)k, k_stride, (const elem_t*)v, v_stride, log_decay, decay_stride,
+               v_scale, v_scale_stride, skip, out, live, stage, state_stride, seg_first, seg_count, slots, heads,
+               heads_per_group, n_keys, n_values, decay_per_channel, write_state, q_scale};
+    const int nr = (n_keys + SCAN_PARTS - 1) / SCAN_PARTS;
+    if (nr <= 8) return launch_scan<8, 16>(a, segments, stream);
+    if (nr <= 16) return launch_scan<16, 16>(a, segments, stream);
+    if (nr <= 32) return launch_scan<32, 16>(a, segments, stream);
+    return launch_scan<64, 8>(a, segments, stream);
+}
+
+}  // extern "C"

@@ -655,6 +655,233 @@ class Kernels:
                _c_int(window or 0), _c_float(scale), _c_int(split_keys), _c_int(max_splits), _p(partial),
                _c_int(TILES_PAIRING[pairing]), _stream()), "attention_tiles")
 
+    # -- a layer whose two branches read the same input ----------------------------------------------
+    @timed("norm", _tensors_work())
+    def add2_rmsnorm2(self, h, d1, d2, w1, w2, out1, out2, eps):
+        """x = h + d1 + d2 (either may be None), written back to h; out1 = rmsnorm(x) * w1 and, when given,
+        out2 = rmsnorm(x) * w2: two norms of one input share its root mean square."""
+        _tensor(h, "h", torch.float32, ndim=2)
+        m, width = h.shape
+        for name, d in (("d1", d1), ("d2", d2)):
+            if d is not None:
+                _tensor(d, name, self.dtype, (m, width))
+        _tensor(w1, "w1", torch.float32, (width,))
+        _tensor(out1, "out1", self.dtype, (m, width))
+        _need((w2 is None) == (out2 is None), "add2_rmsnorm2: the second norm needs a weight and an output")
+        if w2 is not None:
+            _tensor(w2, "w2", torch.float32, (width,))
+            _tensor(out2, "out2", self.dtype, (m, width))
+        fn = self._lib("elementwise").mlr_add2_rmsnorm2
+        _ok(fn(_p(h), _p(d1), _p(d2), _p(w1), _p(w2), _p(out1), _p(out2), _c_int(m), _c_int(width), _c_float(eps),
+               _stream()), "add2_rmsnorm2")
+
+    @timed("norm", _tensors_work())
+    def residual_add2(self, h, d1, d2=None):
+        """h += d1 + d2 (d2 may be None), the sum of the two taken in 32-bit first."""
+        _tensor(h, "h", torch.float32, ndim=2)
+        _tensor(d1, "d1", self.dtype, tuple(h.shape))
+        if d2 is not None:
+            _tensor(d2, "d2", self.dtype, tuple(h.shape))
+        fn = self._lib("elementwise").mlr_residual_add2
+        _ok(fn(_p(h), _p(d1), _p(d2), _c_size_t(h.numel()), _stream()), "residual_add2")
+
+    @timed("activation", _tensors_work())
+    def clamped_glu(self, gate_up, act, limit, slope):
+        """act = g * sigmoid(slope * g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit);
+        gate_up = [gate | up] side by side."""
+        _tensor(gate_up, "gate_up", self.dtype, ndim=2)
+        m, two_f = gate_up.shape
+        _need(two_f % 2 == 0, "gate_up: the width must be even")
+        _tensor(act, "act", self.dtype, (m, two_f // 2))
+        fn = self._lib("elementwise").mlr_clamped_glu
+        _ok(fn(_p(gate_up), _p(act), _c_int(m), _c_int(two_f // 2), _c_float(limit), _c_float(slope), _stream()),
+            "clamped_glu")
+
+    def _columns(self, t, name, dtype, rows, width):
+        """A block of `width` columns of a row-major matrix (a view `x[:, a:b]` or a whole matrix): its row stride."""
+        _need(isinstance(t, torch.Tensor) and t.is_cuda and t.dtype is dtype and t.dim() == 2
+              and tuple(t.shape) == (rows, width) and (t.stride(1) == 1 or width == 1) and t.stride(0) >= width,
+              lambda: f"{name}: expected {dtype} columns [{rows}, {width}] of a row-major matrix on the GPU")
+        return t.stride(0)
+
+    @timed("norm", _tensors_work())
+    def gated_part_norm(self, y, gate, weight, out, part, eps, gate_first, gate_kind="silu"):
+        """y float [rows, width] in parts of `part` values, each over its root mean square, times
+        weight[i % len(weight)]; the activation of `gate` (columns of a matrix) multiplies before the norm
+        (`gate_first`) or after it."""
+        _tensor(y, "y", torch.float32, ndim=2)
+        m, width = y.shape
+        stride = self._columns(gate, "gate", self.dtype, m, width)
+        _tensor(weight, "weight", torch.float32, ndim=1)
+        period = weight.numel()
+        _need(part >= 1 and width % part == 0 and period in (part, width), "gated_part_norm: sizes do not fit")
+        _need(gate_kind in ("silu", "sigmoid"), "gated_part_norm: unknown gate")
+        _tensor(out, "out", self.dtype, (m, width))
+        fn = self._lib("elementwise").mlr_gated_part_norm
+        _ok(fn(_p(y), _p(gate), ctypes.c_long(stride), _p(weight), _p(out), _c_int(m), _c_int(width), _c_int(part),
+               _c_int(period), _c_float(eps), _c_int(1 if gate_first else 0), _c_int(0 if gate_kind == "silu" else 1),
+               _stream()), "gated_part_norm")
+
+    # -- mixers with a state of fixed size ------------------------------------------------------------
+    CONV_MAX_TAPS = 8
+    RECURRENCE_MAX_KEYS = 256
+
+    @timed("conv", _tensors_work())
+    def causal_conv(self, x, weight, bias, out, live, stage, state_offset, slots, positions, silu=True, write_state=True):
+        """out[r, c] = act(bias[c] + sum_j weight[c, j] * input j - (taps - 1) tokens from r), a request's earlier
+        inputs taken from the step's rows or from its state: `live`/`stage` [slots, floats] hold them from
+        `state_offset` on as [taps - 1][channels]."""
+        rows, channels = x.shape
+        xs = self._columns(x, "x", self.dtype, rows, channels)
+        _tensor(weight, "weight", torch.float32, ndim=2)
+        taps = weight.shape[1]
+        _need(weight.shape[0] == channels and 1 <= taps <= self.CONV_MAX_TAPS, "causal_conv: weight must be [channels, 1..8 taps]")
+        if bias is not None:
+            _tensor(bias, "bias", torch.float32, (channels,))
+        os_ = self._columns(out, "out", self.dtype, rows, channels)
+        self._check_state(live, stage, state_offset, (taps - 1) * channels)
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _tensor(positions, "positions", torch.int32, (rows,))
+        fn = self._lib("recurrence").mlr_causal_conv
+        at = state_offset * 4
+        _ok(fn(_p(x), ctypes.c_long(xs), _p(weight), _p(bias), _p(out), ctypes.c_long(os_), _ptr(live.data_ptr() + at),
+               _ptr(stage.data_ptr() + at), ctypes.c_long(live.stride(0)), _p(slots), _p(positions), _c_int(rows),
+               _c_int(channels), _c_int(taps), _c_int(1 if silu else 0), _c_int(1 if write_state else 0), _stream()),
+            "causal_conv")
+
+    @staticmethod
+    def _check_state(live, stage, offset, count):
+        for name, t in (("live", live), ("stage", stage)):
+            _need(isinstance(t, torch.Tensor) and t.is_cuda and t.dtype is torch.float32 and t.dim() == 2
+                  and t.is_contiguous(), f"{name}: the state must be float32 [slots, floats] on the GPU")
+        _need(live.shape == stage.shape and 0 <= offset and offset + count <= live.shape[1],
+              "the state does not hold what the kernel reads and writes")
+
+    @timed("activation", _tensors_work())
+    def gla_log_decay(self, z, bias, out, tau):
+        """out = log(sigmoid(z + bias)^(1 / tau)), 32-bit."""
+        _tensor(z, "z", self.dtype, ndim=2)
+        rows, width = z.shape
+        _tensor(bias, "bias", torch.float32, (width,))
+        _tensor(out, "out", torch.float32, (rows, width))
+        _need(tau > 0, "gla_log_decay: tau must be positive")
+        fn = self._lib("recurrence").mlr_gla_log_decay
+        _ok(fn(_p(z), _p(bias), _p(out), _c_int(rows), _c_int(width), _c_float(1.0 / tau), _stream()), "gla_log_decay")
+
+    @timed("activation", _tensors_work())
+    def mamba_step(self, raw, dt_bias, a_log, dt, log_decay):
+        """dt = softplus(raw + dt_bias), log_decay = -exp(a_log) * dt, 32-bit; raw: columns [rows, heads]."""
+        rows, heads = raw.shape
+        stride = self._columns(raw, "raw", self.dtype, rows, heads)
+        _tensor(dt_bias, "dt_bias", torch.float32, (heads,))
+        _tensor(a_log, "a_log", torch.float32, (heads,))
+        _tensor(dt, "dt", torch.float32, (rows, heads))
+        _tensor(log_decay, "log_decay", torch.float32, (rows, heads))
+        fn = self._lib("recurrence").mlr_mamba_step
+        _ok(fn(_p(raw), ctypes.c_long(stride), _p(dt_bias), _p(a_log), _p(dt), _p(log_decay), _c_int(rows), _c_int(heads),
+               _stream()), "mamba_step")
+
+    @timed("recurrence", _tensors_work())
+    def linear_recurrence(self, q, k, v, log_decay, out, live, stage, state_offset, seg_first, seg_count, segments, slots,
+                          heads, n_keys, n_values, heads_per_group=1, v_scale=None, skip=None, q_scale=1.0,
+                          write_state=True):
+        """Per request of the step and head, from the live state: S_t = diag(exp(log_decay_t)) S_(t-1) + k_t (v_scale_t
+        v_t)^T, out_t = S_t^T (q_scale q_t) + skip[head] v_t.  q, k: columns [rows, (heads / heads_per_group) * n_keys];
+        v: columns [rows, heads * n_values]; log_decay float [rows, heads * n_keys] (a decay per key channel) or
+        [rows, heads] (one per head); v_scale float [rows, heads]; the state [heads][n_keys][n_values] floats from
+        `state_offset` on in a slot's row of `live`/`stage`."""
+        rows = v.shape[0]
+        groups = heads // heads_per_group
+        _need(heads >= 1 and heads_per_group >= 1 and heads % heads_per_group == 0, "linear_recurrence: heads and groups")
+        _need(1 <= n_keys <= self.RECURRENCE_MAX_KEYS, f"linear_recurrence: 1..{self.RECURRENCE_MAX_KEYS} key channels a head")
+        qs = self._columns(q, "q", self.dtype, rows, groups * n_keys)
+        ks = self._columns(k, "k", self.dtype, rows, groups * n_keys)
+        vs = self._columns(v, "v", self.dtype, rows, heads * n_values)
+        _tensor(log_decay, "log_decay", torch.float32, ndim=2)
+        per_channel = log_decay.shape[1] == heads * n_keys and not (n_keys == 1 and False)
+        _need(tuple(log_decay.shape) in ((rows, heads * n_keys), (rows, heads)), "log_decay: [rows, heads * keys] or [rows, heads]")
+        if n_keys == 1:
+            per_channel = True                  # (the two layouts coincide)
+        if v_scale is not None:
+            _tensor(v_scale, "v_scale", torch.float32, (rows, heads))
+        if skip is not None:
+            _tensor(skip, "skip", torch.float32, (heads,))
+        _tensor(out, "out", torch.float32, (rows, heads * n_values))
+        self._check_state(live, stage, state_offset, heads * n_keys * n_values)
+        _tensor(seg_first, "seg_first", torch.int32, (segments,))
+        _tensor(seg_count, "seg_count", torch.int32, (segments,))
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _need(segments <= 65535 * 32 and heads <= 65535, "linear_recurrence: too many requests or heads for the grid")
+        fn = self._lib("recurrence").mlr_linear_recurrence
+        at = state_offset * 4
+        _ok(fn(_p(q), ctypes.c_long(qs), _p(k), ctypes.c_long(ks), _p(v), ctypes.c_long(vs), _p(log_decay),
+               ctypes.c_long(log_decay.shape[1]), _c_int(1 if per_channel else 0), _p(v_scale),
+               ctypes.c_long(heads if v_scale is not None else 0), _p(skip), _c_float(q_scale), _p(out),
+               _ptr(live.data_ptr() + at), _ptr(stage.data_ptr() + at), ctypes.c_long(live.stride(0)), _p(seg_first),
+               _p(seg_count), _p(slots), _c_int(segments), _c_int(heads), _c_int(heads_per_group), _c_int(n_keys),
+               _c_int(n_values), _c_int(1 if write_state else 0), _stream()), "linear_recurrence")
+
+    # -- differential attention -----------------------------------------------------------------------
+    DIFF_MAX_HEAD_DIM = 256
+    DIFF_MAX_VALUE_DIM = 256
+
+    def _check_diff_cache(self, k_pages, v_pages, kv_heads, head_dim, value_dim, page_size):
+        _tensor(k_pages, "k_pages", self.dtype, ndim=4)
+        _tensor(v_pages, "v_pages", self.dtype, ndim=4)
+        pages = k_pages.shape[0]
+        _need(tuple(k_pages.shape) == (pages, kv_heads, page_size, 2 * head_dim), "k_pages: [pages, kv_heads, page, 2 * head_dim]")
+        _need(tuple(v_pages.shape) == (pages, kv_heads, page_size, value_dim), "v_pages: [pages, kv_heads, page, value_dim]")
+
+    @timed("rope_kv", _tensors_work())
+    def diff_kv_write(self, k, v, k_pages, v_pages, block_table, slots, positions, kv_heads, head_dim, value_dim, page_size):
+        """The step's keys (both maps) and values into their pages."""
+        rows = k.shape[0]
+        ks = self._columns(k, "k", self.dtype, rows, kv_heads * 2 * head_dim)
+        vs = self._columns(v, "v", self.dtype, rows, kv_heads * value_dim)
+        self._check_diff_cache(k_pages, v_pages, kv_heads, head_dim, value_dim, page_size)
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _tensor(positions, "positions", torch.int32, (rows,))
+        fn = self._lib("diff_attention").mlr_diff_kv_write
+        _ok(fn(_p(k), ctypes.c_long(ks), _p(v), ctypes.c_long(vs), _p(k_pages), _p(v_pages), _p(block_table),
+               _c_int(block_table.shape[1]), _p(slots), _p(positions), _c_int(rows), _c_int(kv_heads), _c_int(2 * head_dim),
+               _c_int(value_dim), _c_int(page_size), _stream()), "diff_kv_write")
+
+    @staticmethod
+    def diff_partial_numel(rows, q_heads, value_dim, max_splits):
+        return rows * q_heads * 2 * max(1, max_splits) * (value_dim + 2)
+
+    @timed("attention")
+    def diff_attention(self, q, k_pages, v_pages, block_table, slots, positions, gate, out, partial, q_heads, kv_heads,
+                       head_dim, value_dim, page_size, scale, lam, out_scale, eps, softcap=None, temp_coef=0.0,
+                       temp_every=1.0, split_keys=0, max_splits=1):
+        """Differential attention of every token of the step over the cached keys at positions <= its own (the step's
+        own keys are in the cache already): out [rows, q_heads * value_dim], normed, scaled and gated by
+        sigmoid(gate) (gate None: no gate).  q: columns [rows, q_heads * 2 * head_dim]."""
+        rows = q.shape[0]
+        qs = self._columns(q, "q", self.dtype, rows, q_heads * 2 * head_dim)
+        gs = self._columns(gate, "gate", self.dtype, rows, q_heads * value_dim) if gate is not None else 0
+        self._check_diff_cache(k_pages, v_pages, kv_heads, head_dim, value_dim, page_size)
+        _need(head_dim <= self.DIFF_MAX_HEAD_DIM and value_dim <= self.DIFF_MAX_VALUE_DIM,
+              f"diff_attention: head sizes up to {self.DIFF_MAX_HEAD_DIM} (keys) and {self.DIFF_MAX_VALUE_DIM} (values)")
+        _need(q_heads % kv_heads == 0, "diff_attention: q_heads must be a multiple of kv_heads")
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _tensor(positions, "positions", torch.int32, (rows,))
+        _tensor(out, "out", self.dtype, (rows, q_heads * value_dim))
+        _tensor(partial, "partial", torch.float32, ndim=1)
+        max_splits = max(1, max_splits)
+        _need(partial.numel() >= self.diff_partial_numel(rows, q_heads, value_dim, max_splits), "diff_attention: partial too small")
+        _need(max_splits == 1 or (split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0 and max_splits <= MAX_KEY_SPLITS),
+              "diff_attention: key ranges must be multiples of 64 keys, at most 1024 of them")
+        _need(rows * 1 <= 2 ** 31 - 1 and q_heads * 2 <= 65535 and max_splits <= 65535, "diff_attention: grid too large")
+        fn = self._lib("diff_attention").mlr_diff_attention
+        _ok(fn(_p(q), ctypes.c_long(qs), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
+               _p(positions), _p(gate), ctypes.c_long(gs), _p(out), _p(partial), _c_int(rows), _c_int(q_heads),
+               _c_int(kv_heads), _c_int(head_dim), _c_int(value_dim), _c_int(page_size), _c_float(scale),
+               _c_float(softcap or 0.0), _c_float(temp_coef), _c_float(temp_every), _c_float(lam), _c_float(out_scale),
+               _c_float(eps), _c_int(split_keys), _c_int(max_splits), _stream()), "diff_attention")
+
     # -- sampling ----------------------------------------------------------------------------
     def sample_scratch(self, rows):
         """(floats, ints) of scratch memory that `sample` needs for this many rows."""

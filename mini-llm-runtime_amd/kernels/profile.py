@@ -5,7 +5,7 @@ include/minillm/profile.h:11-31; device time src/minillm/cuda/runtime.cpp:176,21
 `Profiler` attached to a `Kernels` object (`Kernels.profiler`) brackets each launch with two events on
 the launch's stream; a profiled runner runs every step eagerly, since events inside a captured graph
 measure nothing.  Classes: embed, norm, gemm (every projection, fused norm and activation
-included), rope_kv, attention (merge of key splits included), activation, sampler, check.  With the
+included), rope_kv, attention (merge of key splits included), conv, recurrence, activation, sampler, check.  With the
 bytes a launch has to move and the flops it has to do (from its operands' shapes; for attention from
 the step's contexts), the report gives GB/s and TFLOP/s per class.
 """
@@ -15,7 +15,7 @@ import functools
 
 import torch
 
-CLASSES = ("embed", "norm", "gemm", "rope_kv", "attention", "activation", "sampler", "check")
+CLASSES = ("embed", "norm", "gemm", "rope_kv", "attention", "conv", "recurrence", "activation", "sampler", "check")
 
 
 class Profiler:

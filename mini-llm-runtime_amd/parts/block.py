@@ -4,7 +4,7 @@ fused with the norm that follows, so a block hands its last output on as `pendin
 adding it itself."""
 from __future__ import annotations
 
-from .registry import Handoff, build_part, register_part
+from .registry import Complete, Handoff, build_part, register_part
 
 
 @register_part("block", "prenorm")
@@ -33,13 +33,86 @@ class PreNormBlock:
             # few rows: every norm is shared between the projection before it (which adds into h and leaves
             # h * weight and partial sums of squares) and the projection after it (which applies the scale)
             hand = pending if isinstance(pending, Handoff) and pending.norm is self.norm1 else \
-                self.norm1.prenorm(ctx, h, None if isinstance(pending, Handoff) else pending)
+                self.norm1.prenorm(ctx, h, None if isinstance(pending, Complete) else pending)
             hand = self.mixer.forward_handoff(ctx, hand, h, self.norm2, cache_id, write_cache)
             return self.ffn.forward_handoff(ctx, hand, h, next_norm if fusable(next_norm) else None)
-        if isinstance(pending, Handoff):                  # h is complete already
+        if isinstance(pending, Complete):                 # h is complete already
             pending = None
         normed = ctx.workspace.get("normed", tuple(h.shape), ctx.dtype)
         self.norm1.forward(ctx, h, pending, normed)
         mixed = self.mixer.forward(ctx, normed, cache_id, write_cache)
         self.norm2.forward(ctx, h, mixed, normed)
         return self.ffn.forward(ctx, normed)
+
+
+@register_part("block", "parallel")
+class ParallelBlock:
+    """Mixer and feed-forward side by side on the same input, each behind a norm of its own:
+    h += mixer(norm1(h)) + ffn(norm2(h)); the sum of the two branches is taken in 32-bit and added to the float
+    residual stream.  `norm2` and `ffn` may be missing (a layer without a feed-forward).  Both norms divide by
+    the same root mean square, so one pass over h serves both (`Kernels.add2_rmsnorm2`), and that pass is the
+    one that adds the branches of the block before: a block ends by norming h for the block that follows
+    (`Normed`) when that one is of this kind too, else it adds its branches itself."""
+    graph_safe = True
+    wants_next_block = True
+
+    def __init__(self, spec):
+        self.norm1 = build_part("norm", spec.norm1)
+        self.mixer = build_part("mixer", spec.mixer)
+        if (spec.ffn is None) != (spec.norm2 is None):
+            raise ValueError("a parallel block has a feed-forward and its norm, or neither")
+        self.norm2 = build_part("norm", spec.norm2) if spec.norm2 is not None else None
+        self.ffn = build_part("ffn", spec.ffn) if spec.ffn is not None else None
+
+    def parts(self):
+        out = {"norm1": self.norm1, "mixer": self.mixer}
+        if self.ffn is not None:
+            out.update(norm2=self.norm2, ffn=self.ffn)
+        return out
+
+    def workspace_plan(self, rows, dtype, limits):
+        width = self.norm1.size
+        return {("normed", dtype): rows * width, ("normed2", dtype): rows * width}
+
+    def _one_pass(self, width):
+        """Whether the block's norms are plain RMSNorms over the whole width with one eps: then they share a pass."""
+        norms = [self.norm1] + ([self.norm2] if self.norm2 is not None else [])
+        return all(getattr(n, "fusable_rmsnorm", False) and n.size == width and n.eps == self.norm1.eps for n in norms)
+
+    def _norm_into(self, ctx, h, d1, d2, x1, x2):
+        """h += d1 + d2 (either may be None); x1 = norm1(h), x2 = norm2(h)."""
+        k = ctx.kernels
+        if self._one_pass(h.shape[1]):
+            k.add2_rmsnorm2(h, d1, d2, self.norm1.weight, self.norm2.weight if self.norm2 is not None else None,
+                            x1, x2 if self.norm2 is not None else None, self.norm1.eps)
+            return
+        if d2 is not None:
+            k.residual_add2(h, d1, d2)
+            d1 = None
+        self.norm1.forward(ctx, h, d1, x1)
+        if self.norm2 is not None:
+            self.norm2.forward(ctx, h, None, x2)
+
+    def forward(self, ctx, h, pending, cache_id, write_cache=True, next_norm=None, next_block=None):
+        from .registry import Normed
+        shape = tuple(h.shape)
+        x1 = ctx.workspace.get("normed", shape, ctx.dtype)
+        x2 = ctx.workspace.get("normed2", shape, ctx.dtype) if self.ffn is not None else None
+        if isinstance(pending, Normed) and pending.norms == ((self.norm1, self.norm2) if self.ffn is not None else (self.norm1,)):
+            x1, x2 = pending.outputs if self.ffn is not None else (pending.outputs[0], None)
+        else:
+            self._norm_into(ctx, h, None if isinstance(pending, Complete) else pending, None, x1, x2)
+        mixed = self.mixer.forward(ctx, x1, cache_id, write_cache)
+        fed = self.ffn.forward(ctx, x2) if self.ffn is not None else None
+        if isinstance(next_block, ParallelBlock) and next_block._one_pass(h.shape[1]):
+            # the branches are added and h is normed for the next block in one pass (its inputs go where this
+            # block's own were: both branches have read them)
+            n1 = ctx.workspace.get("normed", shape, ctx.dtype)
+            n2 = ctx.workspace.get("normed2", shape, ctx.dtype) if next_block.ffn is not None else None
+            next_block._norm_into(ctx, h, mixed, fed, n1, n2)
+            return Normed((next_block.norm1, next_block.norm2) if next_block.ffn is not None else (next_block.norm1,),
+                          (n1, n2) if next_block.ffn is not None else (n1,))
+        if fed is None:
+            return mixed                                  # (one delta: whoever norms next adds it)
+        ctx.kernels.residual_add2(h, mixed, fed)
+        return None

@@ -1,0 +1,123 @@
+"""Differential attention over the paged cache.  Every query head holds two maps: two softmax attentions with
+queries and keys of their own over the same values; the head's output is map 1 - lam * map 2 with
+lam = exp(lq1 . lk1) - exp(lq2 . lk2) + lam_init (one number a layer), divided by its root mean square over the
+value channels, times `out_scale`, times sigmoid of the head's gate; then the output projection.  Query and key
+channels of a map (`head_dim`) and value channels (`value_dim`) are sizes of their own; consecutive query heads
+share a kv head.  There is no rotation: a query's position enters as a factor on it
+(`QueryTemperature`), a score is squashed by `softcap * tanh(score / softcap)`, and position p sees keys 0..p.
+
+Per token the cache keeps the keys of both maps [kv_heads, 2 * head_dim] and the values [kv_heads, value_dim]
+(`PagedSpec`).  q, k, v and the gate are one stacked projection of the mixer's input."""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..cache.manager import PAGE, PagedSpec
+from ..weights.loader import WeightSpec, stacked
+from .registry import PartError, register_part
+
+PARTIAL_CAP = 32 << 20        # floats that the key ranges' partial results of one launch may take at most
+
+
+@register_part("mixer", "diff_attention")
+class DiffAttention:
+    graph_safe = True        # forward launches kernels over the step's device vectors only
+
+    def __init__(self, spec):
+        s = self.spec = spec
+        if s.q_heads % s.kv_heads != 0:
+            raise PartError(f"q_heads {s.q_heads} is no multiple of kv_heads {s.kv_heads}")
+        if not 1 <= s.head_dim <= 256 or not 1 <= s.value_dim <= 256:
+            raise PartError(f"head_dim {s.head_dim} / value_dim {s.value_dim}: the attention kernels take sizes up to 256")
+        if s.gate not in (None, "sigmoid"):
+            raise PartError(f"gate {s.gate!r} is not built (sigmoid or none)")
+        self.q_width, self.k_width = s.q_heads * 2 * s.head_dim, s.kv_heads * 2 * s.head_dim
+        self.v_width, self.o_width = s.kv_heads * s.value_dim, s.q_heads * s.value_dim
+        self.proj = self.o = None
+        self.lam = None
+
+    def weight_specs(self):
+        s = self.spec
+        small = ("normal", 0.0, 0.1)
+        specs = {"q": WeightSpec((self.q_width, s.hidden), stack="qkvg"), "k": WeightSpec((self.k_width, s.hidden), stack="qkvg"),
+                 "v": WeightSpec((self.v_width, s.hidden), stack="qkvg")}
+        if s.gate is not None:
+            specs["g"] = WeightSpec((self.o_width, s.hidden), stack="qkvg")
+        specs["o"] = WeightSpec((s.hidden, self.o_width))
+        for name in ("lq1", "lk1", "lq2", "lk2"):
+            specs[name] = WeightSpec((s.head_dim,), keep_float32=True, init=small)
+        return specs
+
+    def bind(self, weights):
+        s = self.spec
+        self.proj = stacked([weights[n] for n in ("q", "k", "v") + (("g",) if s.gate is not None else ())])
+        self.o = weights["o"]
+        # lam is one number a layer: computed once, in 32-bit, when the weights are bound
+        f = lambda n: weights[n].detach().to("cpu", torch.float32).numpy()
+        one = f("lq1") * f("lk1")
+        two = f("lq2") * f("lk2")
+        import numpy as np
+        self.lam = float(np.exp(one.sum(dtype=np.float32)) - np.exp(two.sum(dtype=np.float32)) + np.float32(s.lam_init))
+
+    def cache_spec(self):
+        s = self.spec
+        return PagedSpec((("k", (s.kv_heads, PAGE, 2 * s.head_dim)), ("v", (s.kv_heads, PAGE, s.value_dim))), None)
+
+    def libraries(self):
+        return ["gemm", "diff_attention"]
+
+    @staticmethod
+    def _splits(max_context, split_keys):
+        """(width of a key range, number of ranges): ranges of `split_keys` keys at absolute positions, whatever
+        the batch; beyond 1024 ranges the width doubles (the merge's limit)."""
+        if split_keys <= 0 or max_context <= split_keys:
+            return 0, 1
+        keys = split_keys
+        while -(-max_context // keys) > 1024:
+            keys *= 2
+        return keys, -(-max_context // keys)
+
+    def workspace_plan(self, rows, dtype, limits):
+        from ..kernels.ops import Kernels
+        s = self.spec
+        _, splits = self._splits(limits["max_length"], limits["split_keys"])
+        per_row = Kernels.diff_partial_numel(1, s.q_heads, s.value_dim, splits)
+        total = self.q_width + self.k_width + self.v_width + (self.o_width if s.gate is not None else 0)
+        return {("diff_proj", dtype): rows * total, ("attn", dtype): rows * self.o_width,
+                ("mixer_out", dtype): rows * s.hidden,
+                ("diff_partial", torch.float32): max(per_row, min(rows * per_row, PARTIAL_CAP))}
+
+    def forward(self, ctx, x, cache_id, write_cache=True):
+        s = self.spec
+        k = ctx.kernels
+        m = x.shape[0]
+        proj = ctx.workspace.get("diff_proj", (m, self.proj.shape[0]), x.dtype)
+        k.gemm(x, self.proj, proj)
+        a = self.q_width
+        b = a + self.k_width
+        c = b + self.v_width
+        q, keys, values = proj[:, :a], proj[:, a:b], proj[:, b:c]
+        gate = proj[:, c:] if s.gate is not None else None
+        view = ctx.cache.paged_view(cache_id)
+        k_pages, v_pages = view.tensors["k"], view.tensors["v"]
+        if write_cache:
+            k.diff_kv_write(keys, values, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, s.kv_heads,
+                            s.head_dim, s.value_dim, view.page_size)
+        attn = ctx.workspace.get("attn", (m, self.o_width), x.dtype)
+        split_keys, splits = self._splits(ctx.max_context, ctx.split_keys)
+        per_row = k.diff_partial_numel(1, s.q_heads, s.value_dim, splits)
+        chunk = max(1, min(m, PARTIAL_CAP // per_row))
+        partial = ctx.workspace.get("diff_partial", (chunk * per_row,), torch.float32)
+        temp = s.q_temperature
+        for r0 in range(0, m, chunk):
+            r1 = min(m, r0 + chunk)
+            k.diff_attention(q[r0:r1], k_pages, v_pages, view.block_table, ctx.slots[r0:r1], ctx.positions[r0:r1],
+                             gate[r0:r1] if gate is not None else None, attn[r0:r1], partial, s.q_heads, s.kv_heads,
+                             s.head_dim, s.value_dim, view.page_size, float(s.scale), self.lam, float(s.out_scale),
+                             float(s.eps), softcap=s.softcap, temp_coef=temp.coef if temp else 0.0,
+                             temp_every=temp.every if temp else 1.0, split_keys=split_keys, max_splits=splits)
+        out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
+        k.gemm(attn, self.o, out)
+        return out

@@ -65,3 +65,47 @@ class SwiGluMlp:
         out = ctx.workspace.get("ffn_out", (m, s.hidden), x.dtype)
         ctx.kernels.gemm(act, self.down, out)
         return out
+
+
+@register_part("ffn", "clamped_glu")
+class ClampedGluMlp:
+    """A gated feed-forward whose branches are clamped: g = min(x Wgate^T, limit), u = clamp(x Wup^T, -limit, limit),
+    out = (g * sigmoid(slope * g) * (u + 1)) Wdown^T.  Gate and up are one stacked projection."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        if not spec.limit > 0:
+            raise PartError("the clamp's limit must be positive")
+        self.spec = spec
+        self.gate_up = None
+        self.down = None
+
+    def weight_specs(self):
+        s = self.spec
+        return {"gate": WeightSpec((s.intermediate, s.hidden), stack="gate_up"),
+                "up": WeightSpec((s.intermediate, s.hidden), stack="gate_up"),
+                "down": WeightSpec((s.hidden, s.intermediate))}
+
+    def bind(self, weights):
+        self.gate_up = stacked([weights["gate"], weights["up"]])
+        self.down = weights["down"]
+
+    def libraries(self):
+        return ["gemm", "elementwise"]
+
+    def workspace_plan(self, rows, dtype, limits):
+        s = self.spec
+        return {("act", dtype): rows * s.intermediate, ("gate_up", dtype): rows * 2 * s.intermediate,
+                ("ffn_out", dtype): rows * s.hidden}
+
+    def forward(self, ctx, x):
+        s = self.spec
+        m = x.shape[0]
+        k = ctx.kernels
+        gate_up = ctx.workspace.get("gate_up", (m, 2 * s.intermediate), x.dtype)
+        k.gemm(x, self.gate_up, gate_up)
+        act = ctx.workspace.get("act", (m, s.intermediate), x.dtype)
+        k.clamped_glu(gate_up, act, float(s.limit), float(s.slope))
+        out = ctx.workspace.get("ffn_out", (m, s.hidden), x.dtype)
+        k.gemm(act, self.down, out)
+        return out

@@ -13,7 +13,7 @@ import torch
 
 from ..config import load_config
 from ..weights.loader import WeightSpec, load_weights
-from .registry import Handoff, PartError, build_part
+from .registry import Complete, PartError, build_part
 
 
 def build_blocks(spec):
@@ -162,12 +162,15 @@ class DecoderModel:
         schedule = self.spec.schedule
         for i, run in enumerate(schedule):
             # (the norm the next run starts with: a block may prepare it while it adds its last output into h)
-            next_norm = self.blocks[schedule[i + 1].layer].norm1 if i + 1 < len(schedule) else None
-            pending = self.blocks[run.layer].forward(ctx, h, pending, run.cache, run.write_cache, next_norm=next_norm)
-            if isinstance(pending, Handoff) and i + 1 == len(schedule):
+            next_block = self.blocks[schedule[i + 1].layer] if i + 1 < len(schedule) else None
+            next_norm = next_block.norm1 if next_block is not None else None
+            block = self.blocks[run.layer]
+            more = {"next_block": next_block} if getattr(block, "wants_next_block", False) else {}
+            pending = block.forward(ctx, h, pending, run.cache, run.write_cache, next_norm=next_norm, **more)
+            if isinstance(pending, Complete) and i + 1 == len(schedule):
                 pending = None                            # (h is complete)
             if status is not None:                        # h + pending is the hidden state after this run
-                k.finite_check(h, None if isinstance(pending, Handoff) else pending, i, status)
+                k.finite_check(h, None if isinstance(pending, Complete) else pending, i, status)
         if ctx.cache is not None and ctx.cache.has_state():
             ctx.cache.commit_state(ctx.segment_slots)     # every layer has run: the staged state becomes live
         r = 0 if want_rows is None else want_rows.numel()

@@ -1,0 +1,178 @@
+"""Mixers that keep a state of fixed size per request instead of keys and values: gated linear attention and
+Mamba-2.  Both run the same recurrence per head,
+    S_t = diag(a_t) S_(t-1) + k_t v_t^T,    o_t = S_t^T q_t       (S: key channels x value channels, 32-bit),
+token by token from the state that earlier steps left (`Kernels.linear_recurrence`); they differ in where q, k,
+v and the decay a come from and in what happens to o.  The state of a request lives in the cache manager's
+slots (`StateSpec`): read from the live rows, written to the staged ones, which become live when every layer of
+the step has run."""
+from __future__ import annotations
+
+import torch
+
+from ..cache.manager import StateSpec
+from ..weights.loader import WeightSpec, stacked
+from .registry import PartError, register_part
+
+WHOLE = 1 << 30          # `StepContext.token_groups(WHOLE)`: every request of the step as one group of rows
+
+
+def _requests(ctx):
+    """(first row, number of rows, how many) of the step's requests, as device vectors."""
+    (first, count, n), _, _ = ctx.token_groups(WHOLE, 0)
+    return first, count, n
+
+
+@register_part("mixer", "gla")
+class GatedLinearAttention:
+    """q = (Wq x) / sqrt(head_dim), k = Wk x, v = Wv x; the decay of key channel i of a head,
+    alpha = sigmoid(z)^(1 / tau) with z = Wa2 (Wa1 x) + b, a low-rank pair; per head the recurrence above; each
+    head's o is RMS-normed over its value channels with one weight vector shared by the heads, the heads are
+    multiplied by silu(Wg x) and projected by Wo."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        s = self.spec = spec
+        if not 1 <= s.head_dim <= 256:
+            raise PartError(f"head_dim {s.head_dim}: the recurrence kernel takes up to 256 key channels a head")
+        if not s.tau > 0:
+            raise PartError("tau must be positive")
+        self.qk_width, self.v_width = s.heads * s.head_dim, s.heads * s.value_dim
+        self.proj = self.a1 = self.a2 = self.a2_bias = self.norm = self.o = None
+
+    def weight_specs(self):
+        s = self.spec
+        rank = s.decay_rank or None              # (None: the file's tensors say)
+        return {"q": WeightSpec((self.qk_width, s.hidden), stack="qkvg"), "k": WeightSpec((self.qk_width, s.hidden), stack="qkvg"),
+                "v": WeightSpec((self.v_width, s.hidden), stack="qkvg"), "g": WeightSpec((self.v_width, s.hidden), stack="qkvg"),
+                "o": WeightSpec((s.hidden, self.v_width)), "norm": WeightSpec((s.value_dim,), keep_float32=True),
+                "a1": WeightSpec((rank, s.hidden)), "a2": WeightSpec((self.qk_width, rank), init=("normal", 0.0, 0.3)),
+                "a2.b": WeightSpec((self.qk_width,), keep_float32=True, init=("normal", 2.0, 1.0))}
+
+    def bind(self, weights):
+        self.proj = stacked([weights[n] for n in ("q", "k", "v", "g")])
+        self.a1, self.a2, self.a2_bias = weights["a1"], weights["a2"], weights["a2.b"]
+        if self.a1.shape[0] != self.a2.shape[1]:
+            raise PartError(f"the decay's two projections do not fit: {tuple(self.a1.shape)} and {tuple(self.a2.shape)}")
+        self.norm, self.o = weights["norm"], weights["o"]
+
+    def cache_spec(self):
+        s = self.spec
+        return StateSpec((s.heads * s.head_dim * s.value_dim,), torch.float32)
+
+    def libraries(self):
+        return ["gemm", "recurrence", "elementwise"]
+
+    def workspace_plan(self, rows, dtype, limits):
+        s = self.spec
+        rank = s.decay_rank or (self.a1.shape[0] if self.a1 is not None else 0)
+        return {("gla_proj", dtype): rows * (2 * self.qk_width + 2 * self.v_width), ("gla_low", dtype): rows * rank,
+                ("gla_z", dtype): rows * self.qk_width, ("log_decay", torch.float32): rows * self.qk_width,
+                ("recurrent_out", torch.float32): rows * self.v_width, ("recurrent_normed", dtype): rows * self.v_width,
+                ("mixer_out", dtype): rows * s.hidden, (f"token_groups_{WHOLE}_0", torch.int32): 2 * rows + 2}
+
+    def forward(self, ctx, x, cache_id, write_cache=True):
+        s = self.spec
+        k = ctx.kernels
+        m = x.shape[0]
+        ws = ctx.workspace
+        proj = ws.get("gla_proj", (m, self.proj.shape[0]), x.dtype)
+        k.gemm(x, self.proj, proj)
+        low = ws.get("gla_low", (m, self.a1.shape[0]), x.dtype)
+        k.gemm(x, self.a1, low)
+        z = ws.get("gla_z", (m, self.qk_width), x.dtype)
+        k.gemm(low, self.a2, z)
+        log_decay = ws.get("log_decay", (m, self.qk_width), torch.float32)
+        k.gla_log_decay(z, self.a2_bias, log_decay, float(s.tau))
+        a, b = self.qk_width, 2 * self.qk_width
+        c = b + self.v_width
+        first, count, n = _requests(ctx)
+        o = ws.get("recurrent_out", (m, self.v_width), torch.float32)
+        k.linear_recurrence(proj[:, :a], proj[:, a:b], proj[:, b:c], log_decay, o, ctx.cache.state_view(cache_id),
+                            ctx.cache.state_stage(cache_id), 0, first, count, n, ctx.slots, s.heads, s.head_dim,
+                            s.value_dim, q_scale=float(s.head_dim) ** -0.5, write_state=write_cache)
+        y = ws.get("recurrent_normed", (m, self.v_width), x.dtype)
+        k.gated_part_norm(o, proj[:, c:], self.norm, y, s.value_dim, float(s.eps), gate_first=False, gate_kind="silu")
+        out = ws.get("mixer_out", (m, s.hidden), x.dtype)
+        k.gemm(y, self.o, out)
+        return out
+
+
+@register_part("mixer", "mamba2")
+class Mamba2:
+    """One input projection laid out [z: inner | x: inner | B: groups * state | C: groups * state | dt: heads] with
+    inner = heads * value_dim; x, B, C pass a short causal convolution per channel (with bias) and silu;
+    dt = softplus(dt + dt_bias); per head (head h reads group h / (heads / groups)) the recurrence above with
+    a = exp(-exp(A_log) dt) on every key channel, k = B, v = dt x, q = C, plus D x; the heads side by side are
+    multiplied by silu(z), RMS-normed in `norm_groups` equal parts, scaled by a weight and projected by Wo.  A
+    request's state is S [heads, state, value_dim] and the convolution's last taps - 1 inputs."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        s = self.spec = spec
+        if s.heads % s.groups != 0:
+            raise PartError(f"heads {s.heads} is no multiple of groups {s.groups}")
+        if not 1 <= s.state <= 256:
+            raise PartError(f"state {s.state}: the recurrence kernel takes up to 256 key channels a head")
+        if not 1 <= s.conv_taps <= 8:
+            raise PartError(f"conv_taps {s.conv_taps}: the convolution kernel takes 1 to 8 taps")
+        self.inner = s.heads * s.value_dim
+        if self.inner % s.norm_groups != 0:
+            raise PartError(f"norm_groups {s.norm_groups} does not divide heads * value_dim = {self.inner}")
+        self.bc = s.groups * s.state
+        self.channels = self.inner + 2 * self.bc
+        self.state_floats = s.heads * s.state * s.value_dim
+        self.w_in = self.conv = self.conv_bias = self.dt_bias = self.a_log = self.skip = self.norm = self.o = None
+
+    def weight_specs(self):
+        s = self.spec
+        vec = lambda n, init=None: WeightSpec((n,), keep_float32=True, init=init)
+        return {"in": WeightSpec((2 * self.inner + 2 * self.bc + s.heads, s.hidden)),
+                "conv": WeightSpec((self.channels, s.conv_taps), keep_float32=True, init=("normal", 0.0, 0.4)),
+                "conv.b": vec(self.channels, ("normal", 0.0, 0.1)), "dt_bias": vec(s.heads, ("uniform", -4.0, 0.0)),
+                "A_log": vec(s.heads, ("uniform", -1.0, 1.5)), "D": vec(s.heads), "norm": vec(self.inner),
+                "o": WeightSpec((s.hidden, self.inner))}
+
+    def bind(self, weights):
+        self.w_in, self.conv, self.conv_bias = weights["in"], weights["conv"], weights["conv.b"]
+        self.dt_bias, self.a_log, self.skip = weights["dt_bias"], weights["A_log"], weights["D"]
+        self.norm, self.o = weights["norm"], weights["o"]
+
+    def cache_spec(self):
+        return StateSpec((self.state_floats + (self.spec.conv_taps - 1) * self.channels,), torch.float32)
+
+    def libraries(self):
+        return ["gemm", "recurrence", "elementwise"]
+
+    def workspace_plan(self, rows, dtype, limits):
+        s = self.spec
+        return {("mamba_proj", dtype): rows * (2 * self.inner + 2 * self.bc + s.heads), ("mamba_conv", dtype): rows * self.channels,
+                ("mamba_dt", torch.float32): rows * s.heads, ("log_decay", torch.float32): rows * s.heads,
+                ("recurrent_out", torch.float32): rows * self.inner, ("recurrent_normed", dtype): rows * self.inner,
+                ("mixer_out", dtype): rows * s.hidden, (f"token_groups_{WHOLE}_0", torch.int32): 2 * rows + 2}
+
+    def forward(self, ctx, x, cache_id, write_cache=True):
+        s = self.spec
+        k = ctx.kernels
+        m = x.shape[0]
+        ws = ctx.workspace
+        proj = ws.get("mamba_proj", (m, self.w_in.shape[0]), x.dtype)
+        k.gemm(x, self.w_in, proj)
+        inner, bc = self.inner, self.bc
+        z, xbc, raw = proj[:, :inner], proj[:, inner:inner + self.channels], proj[:, inner + self.channels:]
+        live, stage = ctx.cache.state_view(cache_id), ctx.cache.state_stage(cache_id)
+        conv = ws.get("mamba_conv", (m, self.channels), x.dtype)
+        k.causal_conv(xbc, self.conv, self.conv_bias, conv, live, stage, self.state_floats, ctx.slots, ctx.positions,
+                      silu=True, write_state=write_cache)
+        dt = ws.get("mamba_dt", (m, s.heads), torch.float32)
+        log_decay = ws.get("log_decay", (m, s.heads), torch.float32)
+        k.mamba_step(raw, self.dt_bias, self.a_log, dt, log_decay)
+        first, count, n = _requests(ctx)
+        y = ws.get("recurrent_out", (m, inner), torch.float32)
+        k.linear_recurrence(conv[:, inner + bc:], conv[:, inner:inner + bc], conv[:, :inner], log_decay, y, live, stage, 0,
+                            first, count, n, ctx.slots, s.heads, s.state, s.value_dim, heads_per_group=s.heads // s.groups,
+                            v_scale=dt, skip=self.skip, write_state=write_cache)
+        normed = ws.get("recurrent_normed", (m, inner), x.dtype)
+        k.gated_part_norm(y, z, self.norm, normed, inner // s.norm_groups, float(s.eps), gate_first=True, gate_kind="silu")
+        out = ws.get("mixer_out", (m, s.hidden), x.dtype)
+        k.gemm(normed, self.o, out)
+        return out

@@ -19,6 +19,9 @@ Interfaces (B = the tokens of a step, E = the model width, T = the engine's elem
                   (the previous block's last output) into h itself, fused with its first norm.
                   `pending` may also be a `Handoff` (h is complete and the first half of a norm is
                   done); a block may return one for `next_norm`, the norm the next block starts with.
+                  Any `Complete` object says that h is complete; a block that does not know its kind
+                  ignores what it carries.  A block class with `wants_next_block = True` is also given
+                  `next_block=` (the block that runs next, or None).
   embed           weight_specs(), bind(), libraries();  forward(ctx) -> the float residual stream [B, E] of
                   the step's tokens (ctx.token_ids);  optional table() -> the [vocab, E] matrix that a tied head
                   may share;  workspace_plan(rows, logits_rows, dtype, limits).
@@ -75,8 +78,21 @@ class Rotation:
     interleaved: bool = False
 
 
+class Complete:
+    """What a block may hand to the next one instead of a pending delta: the residual stream h is complete
+    (nothing is left to be added), and the object carries something that the next block may use or ignore."""
+
+
 @dataclass
-class Handoff:
+class Normed(Complete):
+    """h is complete and normed already for the block that follows: `outputs[i]` is `norms[i]` applied to h (a
+    block that ends with the sum of its branches norms the result for the next block in the same pass)."""
+    norms: tuple
+    outputs: tuple
+
+
+@dataclass
+class Handoff(Complete):
     """A norm shared between the projection before it and the projection after it (few rows, see
     `Kernels.handoff_supported`): the residual stream h is complete (nothing is pending), `x` holds
     T(h * norm.weight) without the rows' scale and `ss` [rows, parts] partial sums of squares of h's rows.

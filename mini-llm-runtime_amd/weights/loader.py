@@ -51,6 +51,11 @@ class WeightSpec:
     optional: bool = False         # e.g. lm_head of a tied model
     stack: Optional[str] = None    # matrices of equal width with the same name here lie row block after
                                    # row block in memory, in the order of their specs (see `stacked`)
+    init: Optional[Tuple] = None   # random-weights mode: ("normal", mean, std) or ("uniform", low, high) instead
+                                   # of the default of its kind
+    # An extent of `shape` may be None: a size that only the file gives (a low rank, say).  The loader puts the
+    # file's extent there before it checks and plans (`resolve_shapes`); the part reads it off the tensor it is
+    # bound to.
 
 
 ALIGN = 256
@@ -163,6 +168,22 @@ def open_model_folder(folder):
     return names, files
 
 
+def resolve_shapes(expected, found):
+    """`expected` with every extent that a spec leaves open (None) taken from the file's tensor of that name
+    (where the file has it with as many extents)."""
+    from dataclasses import replace
+    out = {}
+    for name, spec in expected.items():
+        if any(e is None for e in spec.shape):
+            have = found.get(name)
+            if have is not None and len(have[1]) == len(spec.shape):
+                spec = replace(spec, shape=tuple(int(f) if e is None else e for e, f in zip(spec.shape, have[1])))
+            elif have is None:
+                spec = replace(spec, shape=tuple(0 if e is None else e for e in spec.shape))
+        out[name] = spec
+    return out
+
+
 def check_names(expected, found):
     """expected: {name: WeightSpec}; found: {name: (dtype, shape)}.  Raises one WeightError
     naming everything that is wrong."""
@@ -191,6 +212,7 @@ def load_weights(folder, expected, dtype, device, device_budget_bytes=None, aren
     names, files = open_model_folder(folder)
     try:
         found = {n: f.entries[n] for n, f in names.items()}
+        expected = resolve_shapes(expected, found)
         check_names(expected, found)
         for name in expected:
             if name in found and found[name][0] == torch.bool:

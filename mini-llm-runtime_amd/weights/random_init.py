@@ -28,7 +28,17 @@ def random_tensors(expected, seed, dtype=torch.bfloat16, matrix_std=0.02, norm_s
     def draw(item):
         name, spec = item
         g = _generator(seed, name)
-        if spec.keep_float32:
+        if any(e is None for e in spec.shape):
+            raise ValueError(f"tensor {name}: a size that only a file gives; the configuration must name it for random weights")
+        if spec.init is not None:
+            kind, a, b = spec.init
+            if kind == "normal":
+                t = a + b * torch.randn(spec.shape, generator=g, dtype=torch.float32)
+            elif kind == "uniform":
+                t = a + (b - a) * torch.rand(spec.shape, generator=g, dtype=torch.float32)
+            else:
+                raise ValueError(f"tensor {name}: unknown initialisation {kind!r}")
+        elif spec.keep_float32:
             t = 1.0 + norm_std * torch.randn(spec.shape, generator=g, dtype=torch.float32)
         else:
             t = matrix_std * torch.randn(spec.shape, generator=g, dtype=torch.float32)
@@ -44,7 +54,7 @@ def random_tensors(expected, seed, dtype=torch.bfloat16, matrix_std=0.02, norm_s
 def _numel(shape):
     count = 1
     for extent in shape:
-        count *= int(extent)
+        count *= int(extent or 0)
     return count
 
 
