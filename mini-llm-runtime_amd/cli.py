@@ -55,7 +55,7 @@ def inspect(opts):
     the tensors are the ones the architecture expects (apps/mini_main.cpp:54-69 prints the same of its file)."""
     from .config import load_config
     from .parts.model import expected_tensors
-    from .weights.loader import WeightError, check_names, open_model_folder
+    from .weights.loader import WeightError, check_names, open_model_folder, resolve_shapes
     if not opts.given("--model"):
         raise OptionError("--inspect needs --model")
     folder = opts["--model"]
@@ -63,12 +63,12 @@ def inspect(opts):
     names, files = open_model_folder(folder)
     found = {name: f.entries[name] for name, f in names.items()}
     try:
-        check_names(expected_tensors(config), found)
+        check_names(resolve_shapes(expected_tensors(config), found), found)
         problems = None
     except WeightError as error:
         problems = str(error)
     dimensions = config.to_dict()
-    report = {"architecture": (dimensions.get("architectures") or [type(config).__name__])[0], "dimensions": dimensions,
+    report = {"architecture": getattr(config, "architecture", type(config).__name__), "dimensions": dimensions,
               "files": [os.path.basename(f.path) for f in files],
               "bytes": sum(os.path.getsize(f.path) for f in files), "tensors": len(found),
               "tensor_types": sorted({str(dtype).replace("torch.", "") for dtype, _ in found.values()}),

@@ -184,3 +184,30 @@ def forward(config, tensors, tokens, residuals=None):
             residuals.append(x.copy())
     x = rms_norm(x, np.asarray(tensors["final.norm"], np.float64), eps)
     return x @ np.asarray(tensors["head"], dtype=np.float64).T
+
+
+class PlainTaletar:
+    """A model folder (config.json, model.safetensors) run by the functions above."""
+
+    def __init__(self, folder):
+        import json
+        import os
+
+        import torch
+        from safetensors.torch import load_file
+        with open(os.path.join(folder, "config.json")) as f:
+            self.cfg = json.load(f)
+        self.tensors = {n: (t.to(torch.float64) if t.dtype.is_floating_point else t).numpy()
+                        for n, t in load_file(os.path.join(folder, "model.safetensors")).items()}
+
+    def logits(self, tokens, want=None):
+        rows = forward(self.cfg, self.tensors, tokens)
+        return rows if want is None else rows[np.asarray(want, dtype=np.int64)]
+
+    def greedy(self, prompt, n):
+        tokens, out = list(prompt), []
+        for _ in range(n):
+            t = int(np.argmax(self.logits(tokens, [len(tokens) - 1])[0]))
+            out.append(t)
+            tokens.append(t)
+        return out
