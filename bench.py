@@ -50,7 +50,8 @@ PREFILL_TOKENS = 2048
 class Bench:
     """One model of the given sizes on the GPU and the measurements on it."""
 
-    def __init__(self, size, layers, args):
+    def __init__(self, size, layers, args, sizes=None):
+        """`sizes`: (layers, Qwen3 config keys) in the place of SIZES[size]."""
         import torch
         from mini_llm_runtime_amd.api import parse_dtype
         from mini_llm_runtime_amd.config import config_from_dict
@@ -58,7 +59,7 @@ class Bench:
         self.torch, self.args, self.size = torch, args, size
         self.dtype = parse_dtype(args.dtype)
         self.tag = "bf16" if self.dtype == torch.bfloat16 else "fp32"
-        self.full_layers, sizes = SIZES[size]
+        self.full_layers, sizes = sizes or SIZES[size]
         self.layers = layers if layers > 0 else self.full_layers
         self.cfg = c = config_from_dict(dict(sizes, architectures=["Qwen3ForCausalLM"], num_hidden_layers=self.layers))
         if args.weights == "folder" or (args.weights == "auto" and size == "0.6b"):
@@ -91,6 +92,7 @@ class Bench:
         self.elem = 2 if self.dtype == torch.bfloat16 else 4
         self.weight_bytes = (self.layers * self.layer_params + c.vocab_size * c.hidden_size) * self.elem
         self.kv_bytes_per_token = self.layers * 2 * c.num_key_value_heads * c.head_dim * self.elem
+        self.vocab = c.vocab_size
         self.g = torch.Generator().manual_seed(0)
 
     def close(self):
@@ -115,7 +117,7 @@ class Bench:
                 slab.normal_()
             return
         for s in slots:
-            ids = torch.randint(0, c.vocab_size, (tokens,), generator=self.g).tolist()
+            ids = torch.randint(0, self.vocab, (tokens,), generator=self.g).tolist()
             for at in range(0, tokens, PREFILL_TOKENS):
                 runner.step([Entry(s, ids[at:at + PREFILL_TOKENS], [])])
 
@@ -135,7 +137,7 @@ class Bench:
         runner.warm_up(batch_sizes=[batch], contexts=[context])
         slots = [runner.open_request() for _ in range(batch)]
         self.fill(runner, slots, fill)
-        tokens = torch.randint(0, c.vocab_size, (batch,), generator=self.g).tolist()
+        tokens = torch.randint(0, self.vocab, (batch,), generator=self.g).tolist()
         zeros = [0.0] * batch
 
         def one(tokens):
@@ -171,7 +173,7 @@ class Bench:
         # (the product's defaults: a step of this many tokens is not captured as a graph unless --prefill-graph 1)
         extra = dict(graph_max_tokens=PREFILL_TOKENS) if a.prefill_graph and not a.profile else {}
         runner = self.runner(1, PREFILL_TOKENS, PREFILL_TOKENS, PREFILL_TOKENS, **extra)
-        ids = torch.randint(0, c.vocab_size, (PREFILL_TOKENS,), generator=self.g).tolist()
+        ids = torch.randint(0, self.vocab, (PREFILL_TOKENS,), generator=self.g).tolist()
         times = []
         for i in range(a.prefill_reps):
             s = runner.open_request()
@@ -185,9 +187,7 @@ class Bench:
             runner.close_request(s)
         seconds = statistics.median(times[1:])         # what a request meets; the fastest run beside it
         t = PREFILL_TOKENS
-        flops = 2.0 * t * self.layers * self.layer_params \
-            + 2.0 * t * t * c.num_attention_heads * c.head_dim * self.layers \
-            + 2.0 * c.vocab_size * c.hidden_size
+        flops = self.prefill_flops(t)
         out = dict(value=round(t / seconds, 1), tokens=t, ms=round(seconds * 1e3, 3),
                    ms_best=round(min(times[1:]) * 1e3, 3),
                    frac=round(flops / seconds / MFMA_PEAK[self.tag], 5))
@@ -197,6 +197,12 @@ class Bench:
         del runner
         torch.cuda.empty_cache()
         return out
+
+    def prefill_flops(self, t):
+        c = self.cfg
+        return 2.0 * t * self.layers * self.layer_params \
+            + 2.0 * t * t * c.num_attention_heads * c.head_dim * self.layers \
+            + 2.0 * c.vocab_size * c.hidden_size
 
     def generate_prompt(self, reps=6):
         """A 2048-token prompt through the scheduler with its options left alone but for the slots (`Engine`, as
@@ -408,6 +414,102 @@ class Bench:
                 "mixed_batches": engine.stats["mixed_batches"] - before["mixed_batches"]}
 
 
+# `--only taletar`: layer sizes that resemble a real model's, for a Taletar model whose layers take Mamba-2,
+# differential attention (twice) and gated linear attention in turn, each beside a clamped gated feed-forward, and
+# for the closest model the engine had before, a Qwen3 dense decoder of the same width, heads, feed-forward and
+# number of layers
+DESIGN_SIZES = {
+    "2k": dict(width=2048, ff=5632, vocab=32000, layers=8, heads=16, kv_heads=4,
+               mamba=dict(heads=64, vdim=64, state=128, groups=1, conv=4, norm_groups=1),
+               gla=dict(heads=8, dim=128, vdim=256, rank=16, tau=16.0)),
+    "4k": dict(width=4096, ff=12288, vocab=32000, layers=8, heads=32, kv_heads=8,
+               mamba=dict(heads=128, vdim=64, state=128, groups=8, conv=4, norm_groups=8),
+               gla=dict(heads=16, dim=128, vdim=256, rank=16, tau=16.0)),
+}
+
+
+class TaletarBench(Bench):
+    """A Taletar model of DESIGN_SIZES[size] with random weights drawn on the GPU."""
+
+    def __init__(self, size, args):
+        import torch
+        from mini_llm_runtime_amd.api import parse_dtype
+        from mini_llm_runtime_amd.config import config_from_dict
+        from mini_llm_runtime_amd.parts import DecoderModel, expected_tensors
+        from mini_llm_runtime_amd.weights import random_tensors_on_device
+        d = DESIGN_SIZES[size]
+        self.torch, self.args, self.size = torch, args, size
+        self.dtype = parse_dtype(args.dtype)
+        self.tag = "bf16" if self.dtype == torch.bfloat16 else "fp32"
+        attention = dict(heads=d["heads"], kv_heads=d["kv_heads"], dim=64, vdim=128, diff=0.6, scale=0.125, softcap=50.0,
+                         q_temp=dict(coef=0.3, every=128))
+        mlp = dict(kind="dense", ff=d["ff"], limit=7.0)
+        turn = [("mamba2", d["mamba"]), ("attention", attention), ("attention", attention), ("gla", d["gla"])]
+        self.layers = self.full_layers = d["layers"]
+        layers = [dict(type=turn[i % 4][0], mixer=turn[i % 4][1], mlp=mlp) for i in range(self.layers)]
+        self.cfg = config_from_dict(dict(architecture="Taletar", vocab=d["vocab"], width=d["width"], norm=dict(eps=1e-5),
+                                         layers=layers))
+        self.model = DecoderModel(self.cfg, random_tensors_on_device(expected_tensors(self.cfg), 0, self.dtype, "cuda"),
+                                  self.dtype, "cuda:0")
+        self.weights_from = "drawn on the GPU"
+        self.elem = 2 if self.dtype == torch.bfloat16 else 4
+        self.weight_bytes = self.model.weight_bytes() - d["vocab"] * d["width"] * self.elem     # (the embedding is not read)
+        kinds = [t for t, _ in turn]
+        n_attention = sum(1 for i in range(self.layers) if kinds[i % 4] == "attention")
+        self.kv_bytes_per_token = n_attention * d["kv_heads"] * (2 * 64 + 128) * self.elem
+        # bytes of recurrent state that a decoding request reads and writes a step (32-bit)
+        m, g = d["mamba"], d["gla"]
+        per = {"mamba2": m["heads"] * m["state"] * m["vdim"] * 4 * 2, "gla": g["heads"] * g["dim"] * g["vdim"] * 4 * 2}
+        self.state_bytes = sum(per.get(kinds[i % 4], 0) for i in range(self.layers))
+        self.matrix_params = (self.model.weight_bytes() // self.elem) - 2 * d["vocab"] * d["width"]
+        self.attention_flops = lambda t: n_attention * 2.0 * t * t * d["heads"] * (2 * 64 + 2 * 128)
+        self.vocab = d["vocab"]
+        self.g = torch.Generator().manual_seed(0)
+
+    def prefill_flops(self, t):
+        d = DESIGN_SIZES[self.size]
+        return 2.0 * t * self.matrix_params + self.attention_flops(t) + 2.0 * d["vocab"] * d["width"]
+
+    def decode_point(self, batch, steps, warmup, context=None):
+        seconds, mean_context, report = self.decode(batch, steps, warmup, context)
+        step_bytes = self.weight_bytes + batch * (mean_context * self.kv_bytes_per_token + self.state_bytes)
+        return dict(tok_s=round(batch * steps / seconds, 1), ms=round(seconds / steps * 1e3, 4),
+                    frac=round(step_bytes / (seconds / steps) / HBM_PEAK, 5)), step_bytes, report
+
+
+def design_block(args):
+    """Prefill (2048 tokens in one step) and decode (batch 8 and 64 behind --context tokens) of the Taletar sizes
+    beside a Qwen3 dense model of equal width, heads, feed-forward and layers; then the same steps once more with
+    events around every launch: milliseconds per kernel class."""
+    import copy
+    out = {}
+    for size in (args.design_sizes.split(",") if args.design_sizes else list(DESIGN_SIZES)):
+        d = DESIGN_SIZES[size]
+        dense = (d["layers"], dict(hidden_size=d["width"], num_attention_heads=d["heads"], num_key_value_heads=d["kv_heads"],
+                                   head_dim=128, intermediate_size=d["ff"], vocab_size=d["vocab"],
+                                   max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1000000.0,
+                                   tie_word_embeddings=False))
+        block = {}
+        for name, make in (("taletar", lambda a: TaletarBench(size, a)), ("qwen3_dense", lambda a: Bench(size, 0, a, sizes=dense))):
+            plain_args, profiled = copy.copy(args), copy.copy(args)
+            plain_args.profile, plain_args.weights = False, "gpu"
+            profiled.profile, profiled.weights, profiled.prefill_reps = True, "gpu", 3
+            bench = make(plain_args)
+            row = {"weight_gb": round(bench.weight_bytes / 1e9, 3), "prefill": bench.prefill()}
+            few = (max(8, args.steps // 2), max(2, args.warmup // 2))
+            for batch in (8, 64):
+                row[f"decode_b{batch}"] = bench.decode_point(batch, *few, context=args.context)[0]
+            bench.args = profiled
+            row["prefill_classes_ms"] = {k: v["ms"] / 2 for k, v in bench.prefill()["profile"].items() if isinstance(v, dict)}
+            _, _, report = bench.decode_point(8, 8, 2, context=args.context)
+            row["decode_b8_classes_ms"] = {k: round(v["ms"] / 8, 4) for k, v in report.items() if isinstance(v, dict)}
+            block[name] = row
+            bench.close()
+            del bench
+        out[size] = block
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -429,11 +531,12 @@ def main():
                          "tensors drawn on the GPU; auto: folder for the 0.6B sizes, gpu for the larger ones")
     ap.add_argument("--warm-up", type=int, default=0,
                     help="--only engine: 1 captures the decoding steps (Engine.warm_up) before the first burst")
-    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prompt", "engine", "mixed"],
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prompt", "engine", "mixed", "taletar"],
                     help="profiling aid: run just the decode steps, just the prefill or just the mixed step; prompt: one "
                          "prompt of --context tokens in portions of 2048; engine: the "
                          "scheduler over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "
                          "batch slots), printed as one line of its own")
+    ap.add_argument("--design-sizes", default="", help="--only taletar: which of its sizes (2k, 4k; default both)")
     ap.add_argument("--library", type=int, default=1,
                     help="0: every matrix product on the hand-written kernels, none in the vendor library")
     ap.add_argument("--split-keys", type=int, default=256, help="the smallest range of keys of one attention workgroup")
@@ -457,6 +560,9 @@ def main():
     if not args.tune:
         from mini_llm_runtime_amd.kernels import build
         build.load("library_gemm").mlr_library_gemm_tuning(0)
+    if args.only == "taletar":
+        print(json.dumps({"taletar_sizes": design_block(args), "context": args.context, "dtype": args.dtype}))
+        return 0
     bench = Bench(args.size, args.layers, args)
     c = bench.cfg
     if args.only == "prefill":

@@ -51,6 +51,30 @@ def random_tensors(expected, seed, dtype=torch.bfloat16, matrix_std=0.02, norm_s
         return dict(pool.map(draw, todo))              # (in the order of `expected`)
 
 
+def random_tensors_on_device(expected, seed, dtype, device, matrix_std=0.02, norm_std=0.1):
+    """The same kinds of tensors drawn on the device itself (other values than `random_tensors` gives for the
+    seed): a model of many gigabytes without the trip through a file.  32-bit vectors stay float32, the rest gets
+    `dtype`, as the loader would place them."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    out = {}
+    for name, spec in expected.items():
+        if spec.optional:
+            continue
+        if any(e is None for e in spec.shape):
+            raise ValueError(f"tensor {name}: a size that only a file gives; the configuration must name it for random weights")
+        kind = torch.float32 if spec.keep_float32 else dtype
+        if spec.init is not None and spec.init[0] == "uniform":
+            t = torch.rand(spec.shape, generator=g, device=device, dtype=torch.float32)
+            t = t.mul_(spec.init[2] - spec.init[1]).add_(spec.init[1])
+        else:
+            mean, std = (spec.init[1], spec.init[2]) if spec.init is not None else (1.0, norm_std) if spec.keep_float32 \
+                else (0.0, matrix_std)
+            t = torch.randn(spec.shape, generator=g, device=device, dtype=kind).mul_(std).add_(mean)
+        out[name] = t.to(kind)
+    return out
+
+
 def _numel(shape):
     count = 1
     for extent in shape:
