@@ -7,15 +7,23 @@
 // temp(p) = 1 + coef * ln(floor((p + 1) / every) + 1) growing with its position p; then, with a cap,
 // score <- cap * tanh(score / cap); position p sees the keys 0 .. p.  All of this is 32-bit.
 //
-// Cache of one layer: keys pages[num_pages][kv_heads][page_size][2 * head_dim], values
-// pages[num_pages][kv_heads][page_size][value_dim].  Query head h reads kv head h / (q_heads / kv_heads).
+// Cache of one layer: keys pages[num_pages][kv_heads][page_size][2 * head_dim]; values transposed within a
+// page, pages[num_pages][kv_heads][value_dim][page_size], so that the keys of one channel lie side by side (the
+// operand layout of the matrix cores for probabilities x values).  Query head h reads kv head
+// h / (q_heads / kv_heads).
 //
 // `diff_attention_partial_kernel`: one wavefront per (token, head and map, key range).  Key ranges are
 // [s * split_keys, (s + 1) * split_keys) in absolute positions and tiles of 64 keys start at multiples of 64, so
 // the order of a token's sums follows from its own position alone, never from the batch around it or from how
 // its request was cut into steps.  It leaves (max, sum, weighted values) per range;
 // `diff_attention_combine_kernel` merges the ranges in ascending order, takes the difference of the maps, norms
-// and gates.
+// and gates.  Both serve the float engine for every token, and the bfloat16 engine for single tokens and short
+// portions (and for the sizes that the matrix-core kernel does not take).
+//
+// `diff_attention_tiles_kernel` (bfloat16): prompt portions on the matrix cores.  A workgroup takes up to 64
+// consecutive tokens of one request and up to four query heads of one kv head; a wavefront 16 tokens of one head,
+// both maps.  Keys and values are staged once per workgroup through LDS in tiles of 32 keys and serve both maps of
+// all its heads; the head's epilogue (difference, norm, gate) runs in registers.
 #include "common.h"
 
 #define TILE_KEYS 64
@@ -32,7 +40,16 @@ struct DiffArgs {
     float* partial;                            // [rows, q_heads * 2, max_splits, value_dim + 2]
     int max_blocks, q_heads, kv_heads, head_dim, value_dim, page_size, split_keys, max_splits;
     float scale, softcap, temp_coef, temp_every, lam, out_scale, eps;
+    // which rows: null: blockIdx.x is the batch row; else blockIdx.x = group * group_tokens + i stands for row
+    // group_first[group] + i while i < group_count[group] (partial results are indexed by blockIdx.x)
+    const int32_t* group_first; const int32_t* group_count; int group_tokens;
 };
+
+__device__ __forceinline__ int diff_row(const DiffArgs& a) {
+    if (a.group_first == nullptr) return blockIdx.x;
+    const int g = blockIdx.x / a.group_tokens, i = blockIdx.x % a.group_tokens;
+    return i < a.group_count[g] ? a.group_first[g] + i : -1;
+}
 
 // Writes the step's keys [kv_heads][2 * head_dim] and values [kv_heads][value_dim] into their pages.
 __global__ void diff_kv_write_kernel(const elem_t* __restrict__ k, long k_stride, const elem_t* __restrict__ v, long v_stride,
@@ -51,7 +68,7 @@ __global__ void diff_kv_write_kernel(const elem_t* __restrict__ k, long k_stride
     }
     for (int i = threadIdx.x; i < kv_heads * value_dim; i += blockDim.x) {
         const int g = i / value_dim, d = i % value_dim;
-        v_pages[(((size_t)page * kv_heads + g) * page_size + at) * value_dim + d] = v[(size_t)m * v_stride + i];
+        v_pages[(((size_t)page * kv_heads + g) * value_dim + d) * page_size + at] = v[(size_t)m * v_stride + i];
     }
 }
 
@@ -65,7 +82,8 @@ __global__ __launch_bounds__(64) void diff_attention_partial_kernel(DiffArgs a) 
     __shared__ float p_lds[TILE_KEYS];
     __shared__ long long k_off[TILE_KEYS];
     __shared__ long long v_off[TILE_KEYS];
-    const int m = blockIdx.x, hm = blockIdx.y, split = blockIdx.z;
+    const int m = diff_row(a), hm = blockIdx.y, split = blockIdx.z;
+    if (m < 0) return;
     const int head = hm >> 1, map = hm & 1;
     const int lane = threadIdx.x;
     const int D = a.head_dim, V = a.value_dim;
@@ -76,7 +94,7 @@ __global__ __launch_bounds__(64) void diff_attention_partial_kernel(DiffArgs a) 
         kbegin = split * a.split_keys;
         kend = min(kend, (split + 1) * a.split_keys);
     }
-    float* dst = a.partial + (((size_t)m * a.q_heads * 2 + hm) * a.max_splits + split) * (V + 2);
+    float* dst = a.partial + (((size_t)blockIdx.x * a.q_heads * 2 + hm) * a.max_splits + split) * (V + 2);
     if (kbegin >= kend) return;                // (a range beyond the token: the merge does not read it)
     for (int i = lane; i < D; i += 64) q_lds[i] = to_float(a.q[(size_t)m * a.q_stride + (size_t)hm * D + i]);
     const float factor = a.scale * query_temperature(pos, a.temp_coef, a.temp_every);
@@ -93,9 +111,9 @@ __global__ __launch_bounds__(64) void diff_attention_partial_kernel(DiffArgs a) 
                 const int block = kp / a.page_size;
                 const int page = block < a.max_blocks ? table[block] : -1;
                 if (page >= 0) {
-                    const long long row = ((long long)page * a.kv_heads + kvh) * a.page_size + kp % a.page_size;
-                    ko = row * (2 * D) + (long long)map * D;
-                    vo = row * V;
+                    const long long head_page = (long long)page * a.kv_heads + kvh;
+                    ko = (head_page * a.page_size + kp % a.page_size) * (2 * D) + (long long)map * D;
+                    vo = head_page * V * a.page_size + kp % a.page_size;
                 }
             }
             k_off[lane] = ko;
@@ -137,7 +155,7 @@ __global__ __launch_bounds__(64) void diff_attention_partial_kernel(DiffArgs a) 
 #pragma unroll
             for (int i = 0; i < MAX_V_REGS; ++i) {
                 const int c = lane + 64 * i;
-                if (c < V) acc[i] += pk * to_float(a.v_pages[off + c]);
+                if (c < V) acc[i] += pk * to_float(a.v_pages[off + (long long)c * a.page_size]);
             }
         }
     }
@@ -156,13 +174,14 @@ __global__ __launch_bounds__(64) void diff_attention_partial_kernel(DiffArgs a) 
 __global__ __launch_bounds__(64) void diff_attention_combine_kernel(DiffArgs a) {
     __shared__ float w_lds[COMBINE_MAX_SPLITS];
     __shared__ float l_lds[COMBINE_MAX_SPLITS];
-    const int m = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const int m = diff_row(a), head = blockIdx.y, lane = threadIdx.x;
+    if (m < 0) return;
     const int V = a.value_dim;
     const int pos = a.positions[m];
     const int n = a.max_splits > 1 ? min(a.max_splits - 1, pos / a.split_keys) + 1 : 1;
     float maps[2][MAX_V_REGS];
     for (int map = 0; map < 2; ++map) {
-        const float* base = a.partial + ((size_t)m * a.q_heads * 2 + head * 2 + map) * a.max_splits * (V + 2);
+        const float* base = a.partial + ((size_t)blockIdx.x * a.q_heads * 2 + head * 2 + map) * a.max_splits * (V + 2);
         float gmax = -INFINITY;
         __syncthreads();
         for (int s = lane; s < n; s += 64) {
@@ -214,6 +233,245 @@ __global__ __launch_bounds__(64) void diff_attention_combine_kernel(DiffArgs a) 
     }
 }
 
+#if MLR_BF16
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+#define TKEYS 32
+
+// NCH: ceil(head_dim / 32) chunks of 32 channels a map; NDB: blocks of 16 value channels (value_dim <= 16 NDB).
+// head_dim and value_dim multiples of 16, the page size a multiple of 8.
+template <int NCH, int NDB>
+__global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffArgs a, const int32_t* __restrict__ group_row0,
+                                                                   const int32_t* __restrict__ group_ntok,
+                                                                   int heads_per_wg, int token_blocks) {
+    constexpr int KPITCH = 2 * 32 * NCH + 8;          // elements per key row in LDS (both maps)
+    constexpr int VPITCH = TKEYS + 4;                 // elements per value channel row in LDS
+    __shared__ __attribute__((aligned(16))) __bf16 k_lds[TKEYS * KPITCH];
+    __shared__ __attribute__((aligned(16))) __bf16 v_lds[16 * NDB * VPITCH];
+    const int D = a.head_dim, V = a.value_dim, P = a.page_size;
+    const int g = a.q_heads / a.kv_heads;
+    const int head_sets = (g + heads_per_wg - 1) / heads_per_wg;
+    const int grp = blockIdx.x, kvh = blockIdx.y / head_sets, head_set = blockIdx.y % head_sets;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 15, b = lane >> 4;
+    const int row0 = group_row0[grp], ntok = group_ntok[grp];
+    const int slot = a.slots[row0], pos0 = a.positions[row0];
+    const int hh = head_set * heads_per_wg + wave % heads_per_wg;         // head within the kv head's set
+    const int tblock = wave / heads_per_wg;
+    const int head = kvh * g + hh;
+    const int tok = tblock * 16 + col;
+    const bool wave_active = tblock < token_blocks && hh < g && tblock * 16 < ntok;
+    const bool col_valid = wave_active && tok < ntok;
+    const int pos = pos0 + tok;
+    const int kend_c = col_valid ? pos + 1 : 0;       // keys this column sees: [0, kend_c)
+    const int ke = pos0 + ntok;                       // keys the workgroup walks: [0, ke)
+    const int wave_hi = wave_active ? pos0 + min(ntok, tblock * 16 + 16) : 0;
+    const int wave_first_kend = pos0 + tblock * 16 + 1;
+    const __bf16* q = reinterpret_cast<const __bf16*>(a.q);
+    const __bf16* kp_base = reinterpret_cast<const __bf16*>(a.k_pages);
+    const __bf16* vp_base = reinterpret_cast<const __bf16*>(a.v_pages);
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int32_t* table = a.block_table + (size_t)slot * a.max_blocks;
+
+    bf16x8 qf[2][NCH];
+#pragma unroll
+    for (int map = 0; map < 2; ++map)
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int d0 = 32 * c + 8 * b;
+            qf[map][c] = zero8;
+            if (col_valid && d0 < D)
+                qf[map][c] = *reinterpret_cast<const bf16x8*>(q + (size_t)(row0 + tok) * a.q_stride + (size_t)(head * 2 + map) * D + d0);
+        }
+    // scores in the base-2 domain; the cap as cap * tanh(x / cap) with tanh(y) = 1 - 2 / (exp(2 y) + 1)
+    const float LOG2E = 1.44269504088896340736f;
+    const float factor = a.scale * query_temperature(pos, a.temp_coef, a.temp_every);
+    const bool capped = a.softcap > 0.f;
+    const float pre = capped ? factor * (2.0f * LOG2E / a.softcap) : factor * LOG2E;
+    const float cap2 = a.softcap * LOG2E;
+    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+    floatx4 o[2][NDB];
+#pragma unroll
+    for (int map = 0; map < 2; ++map)
+#pragma unroll
+        for (int i = 0; i < NDB; ++i) o[map][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const int k_chunks = TKEYS * (2 * D / 8);         // 16-byte chunks of a key tile: key-major
+    const int v_chunks = V * (TKEYS / 8);             // of a value tile: channel-major, 8 keys each
+    // with key ranges: this workgroup walks [split * split_keys, (split + 1) * split_keys) (multiples of 32) and
+    // leaves partial results for the merge
+    const int split = blockIdx.z;
+    const int k_lo = a.max_splits > 1 ? split * a.split_keys : 0;
+    const int k_hi = a.max_splits > 1 ? min(ke, (split + 1) * a.split_keys) : ke;
+    for (int tb = k_lo; tb < k_hi; tb += TKEYS) {
+        __syncthreads();                              // the tile before has been read
+        for (int ci = threadIdx.x; ci < k_chunks; ci += 256) {
+            const int key = ci / (2 * D / 8), c8 = ci % (2 * D / 8);
+            const int kp = tb + key;
+            bf16x8 kv = zero8;
+            if (kp < k_hi) {
+                const int block = kp / P;
+                const int page = block < a.max_blocks ? table[block] : -1;
+                if (page >= 0)
+                    kv = *reinterpret_cast<const bf16x8*>(kp_base + (((size_t)page * a.kv_heads + kvh) * P + kp % P) * (2 * D) + 8 * c8);
+            }
+            // (map m's channel d goes to column m * 32 NCH + d, so that both maps start a row of chunks)
+            const int ch = 8 * c8, map = ch >= D ? 1 : 0;
+            *reinterpret_cast<bf16x8*>(&k_lds[key * KPITCH + map * 32 * NCH + (ch - map * D)]) = kv;
+        }
+        for (int ci = threadIdx.x; ci < v_chunks; ci += 256) {
+            const int d = ci >> 2, q4 = ci & 3;
+            const int kp = tb + 8 * q4;
+            bf16x8 v = zero8;
+            if (kp < k_hi) {
+                const int block = kp / P;
+                const int page = block < a.max_blocks ? table[block] : -1;
+                if (page >= 0)
+                    v = *reinterpret_cast<const bf16x8*>(vp_base + (((size_t)page * a.kv_heads + kvh) * V + d) * P + kp % P);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)           // keys that are not written yet count as zero
+                    if (kp + e >= k_hi) v[e] = (__bf16)0.f;
+            }
+            *reinterpret_cast<bf16x4*>(&v_lds[d * VPITCH + 8 * q4]) = bf16x4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<bf16x4*>(&v_lds[d * VPITCH + 8 * q4 + 4]) = bf16x4{v[4], v[5], v[6], v[7]};
+        }
+        __syncthreads();
+        if (!wave_active || tb >= wave_hi) continue;
+        const bool interior = tb + TKEYS <= wave_first_kend;
+#pragma unroll
+        for (int map = 0; map < 2; ++map) {
+            floatx4 s[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                s[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+                    bf16x8 kf = zero8;                // (channels at and beyond head_dim were never staged)
+                    if (32 * c + 8 * b < D)
+                        kf = *reinterpret_cast<const bf16x8*>(&k_lds[(16 * j + col) * KPITCH + map * 32 * NCH + 32 * c + 8 * b]);
+                    s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[map][c], s[j], 0, 0, 0);
+                }
+            }
+            float sv[2][4];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float x = s[j][r] * pre;
+                    if (capped) {
+                        const float e = __builtin_amdgcn_exp2f(x);                    // exp(2 s / cap)
+                        x = cap2 - 2.0f * cap2 * __builtin_amdgcn_rcpf(e + 1.0f);
+                    }
+                    const int key = tb + 16 * j + 4 * b + r;
+                    sv[j][r] = (interior || key < kend_c) ? x : -INFINITY;
+                }
+            float tile_max = fmaxf(fmaxf(fmaxf(sv[0][0], sv[0][1]), fmaxf(sv[0][2], sv[0][3])),
+                                   fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLR_WAVE));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLR_WAVE));
+            if (__builtin_amdgcn_ballot_w64(tile_max > m_run[map]) != 0) {
+                const float m_new = fmaxf(m_run[map], tile_max);
+                const float corr = m_new > -INFINITY ? __builtin_amdgcn_exp2f(m_run[map] - m_new) : 1.f;
+                l_run[map] *= corr;
+#pragma unroll
+                for (int db = 0; db < NDB; ++db) o[map][db] *= corr;
+                m_run[map] = m_new;
+            }
+            const float m_use = fmaxf(m_run[map], -1e30f);
+            bf16x8 pf;
+            float psum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float p = __builtin_amdgcn_exp2f(sv[j][r] - m_use);
+                    psum += p;
+                    pf[4 * j + r] = (__bf16)p;
+                }
+            l_run[map] += psum;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+                if (16 * db >= V) break;
+                const __bf16* vrow = &v_lds[(16 * db + col) * VPITCH];
+                const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vrow + 4 * b);
+                const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vrow + 16 + 4 * b);
+                const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                o[map][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[map][db], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int map = 0; map < 2; ++map) {
+        l_run[map] += __shfl_xor(l_run[map], 16, MLR_WAVE);
+        l_run[map] += __shfl_xor(l_run[map], 32, MLR_WAVE);
+    }
+    if (a.max_splits > 1) {
+        // (max, sum, weighted values) of this key range, the maximum back in the natural domain
+        if (!col_valid) return;
+        const size_t place = (size_t)grp * a.group_tokens + tok;
+#pragma unroll
+        for (int map = 0; map < 2; ++map) {
+            float* dst = a.partial + ((place * a.q_heads * 2 + head * 2 + map) * a.max_splits + split) * (V + 2);
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+                if (16 * db >= V) break;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) dst[16 * db + 4 * b + r] = o[map][db][r];
+            }
+            if (b == 0) {
+                dst[V] = m_run[map] * 0.69314718055994530942f;
+                dst[V + 1] = l_run[map];
+            }
+        }
+        return;
+    }
+    // the head's epilogue: lane (col, b) holds channels 16 db + 4 b + r of its column
+    const float inv1 = l_run[0] != 0.f ? 1.0f / l_run[0] : 0.f, inv2 = l_run[1] != 0.f ? 1.0f / l_run[1] : 0.f;
+    float ss = 0.f;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+        if (16 * db >= V) break;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float d = o[0][db][r] * inv1 - a.lam * (o[1][db][r] * inv2);
+            o[0][db][r] = d;
+            ss += d * d;
+        }
+    }
+    ss += __shfl_xor(ss, 16, MLR_WAVE);
+    ss += __shfl_xor(ss, 32, MLR_WAVE);
+    if (!col_valid) return;
+    const float unit = a.out_scale / sqrtf(ss / (float)V + a.eps);
+    __bf16* dst = reinterpret_cast<__bf16*>(a.out) + ((size_t)(row0 + tok) * a.q_heads + head) * V;
+    const __bf16* gate = a.gate ? reinterpret_cast<const __bf16*>(a.gate) + (size_t)(row0 + tok) * a.gate_stride + (size_t)head * V : nullptr;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+        if (16 * db >= V) break;
+        bf16x4 w4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float y = o[0][db][r] * unit;
+            if (gate) y *= 1.0f / (1.0f + __expf(-(float)gate[16 * db + 4 * b + r]));
+            w4[r] = (__bf16)y;
+        }
+        *reinterpret_cast<bf16x4*>(dst + 16 * db + 4 * b) = w4;
+    }
+}
+
+template <int NCH>
+static int launch_tiles(const DiffArgs& a, const int32_t* row0, const int32_t* ntok, int groups, int hpw, int tbw,
+                        hipStream_t stream) {
+    const int g = a.q_heads / a.kv_heads;
+    dim3 grid(groups, a.kv_heads * ((g + hpw - 1) / hpw), a.max_splits);
+    const int ndb = (a.value_dim + 15) / 16;
+    if (ndb <= 2) diff_attention_tiles_kernel<NCH, 2><<<grid, 256, 0, stream>>>(a, row0, ntok, hpw, tbw);
+    else if (ndb <= 4) diff_attention_tiles_kernel<NCH, 4><<<grid, 256, 0, stream>>>(a, row0, ntok, hpw, tbw);
+    else diff_attention_tiles_kernel<NCH, 8><<<grid, 256, 0, stream>>>(a, row0, ntok, hpw, tbw);
+    return (int)hipGetLastError();
+}
+#endif
+
 extern "C" {
 
 int mlr_diff_kv_write(const void* k, long k_stride, const void* v, long v_stride, void* k_pages, void* v_pages,
@@ -230,7 +488,10 @@ int mlr_diff_attention(const void* q, long q_stride, const void* k_pages, const 
                        int max_blocks, const int32_t* slots, const int32_t* positions, const void* gate, long gate_stride,
                        void* out, float* partial, int rows, int q_heads, int kv_heads, int head_dim, int value_dim,
                        int page_size, float scale, float softcap, float temp_coef, float temp_every, float lam,
-                       float out_scale, float eps, int split_keys, int max_splits, hipStream_t stream) {
+                       float out_scale, float eps, int split_keys, int max_splits, const int32_t* group_first,
+                       const int32_t* group_count, int groups, int group_tokens, hipStream_t stream) {
+    // (with groups: `rows` = groups * group_tokens places, of which those beyond a group's count stay idle)
+    if (group_first != nullptr) rows = groups * group_tokens;
     if (rows <= 0) return 0;
     if (head_dim > 256 || value_dim > 64 * MAX_V_REGS || q_heads % kv_heads != 0 || partial == nullptr) return -1;
     if (max_splits < 1) max_splits = 1;
@@ -238,12 +499,52 @@ int mlr_diff_attention(const void* q, long q_stride, const void* k_pages, const 
     if (temp_coef != 0.f && !(temp_every > 0.f)) return -3;
     DiffArgs a{(const elem_t*)q, q_stride, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots, positions,
                (const elem_t*)gate, gate_stride, (elem_t*)out, partial, max_blocks, q_heads, kv_heads, head_dim, value_dim,
-               page_size, split_keys, max_splits, scale, softcap, temp_coef, temp_every, lam, out_scale, eps};
+               page_size, split_keys, max_splits, scale, softcap, temp_coef, temp_every, lam, out_scale, eps,
+               group_first, group_count, group_tokens};
     diff_attention_partial_kernel<<<dim3(rows, q_heads * 2, max_splits), 64, 0, stream>>>(a);
     int err = (int)hipGetLastError();
     if (err != 0) return err;
     diff_attention_combine_kernel<<<dim3(rows, q_heads), 64, 0, stream>>>(a);
     return (int)hipGetLastError();
+}
+
+// Groups of consecutive tokens of one request on the matrix cores (bfloat16): prompt portions in groups of up to
+// 16 * (4 / min(4, q_heads / kv_heads)) tokens, single tokens and short portions in smaller ones.  `group_tokens`:
+// the most tokens of a group.  With max_splits > 1 every group's keys are cut into ranges of split_keys (a
+// multiple of 64) whose partial results [groups * group_tokens, q_heads * 2, max_splits, value_dim + 2] are merged
+// by the kernel that also serves the scalar path.  Returns -10 where the sizes are not taken.
+int mlr_diff_attention_tiles(const void* q, long q_stride, const void* k_pages, const void* v_pages,
+                             const int32_t* block_table, int max_blocks, const int32_t* slots, const int32_t* positions,
+                             const void* gate, long gate_stride, void* out, float* partial, const int32_t* group_row0,
+                             const int32_t* group_ntok, int groups, int group_tokens, int q_heads, int kv_heads,
+                             int head_dim, int value_dim, int page_size, float scale, float softcap, float temp_coef,
+                             float temp_every, float lam, float out_scale, float eps, int split_keys, int max_splits,
+                             hipStream_t stream) {
+#if MLR_BF16
+    if (groups <= 0) return 0;
+    if (head_dim % 16 != 0 || head_dim > 128 || value_dim % 16 != 0 || value_dim > 128 || page_size % 8 != 0 ||
+        q_heads % kv_heads != 0 || q_stride % 8 != 0 || (gate != nullptr && gate_stride % 4 != 0)) return -10;
+    if (max_splits < 1) max_splits = 1;
+    if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % TILE_KEYS != 0 ||
+                           max_splits > COMBINE_MAX_SPLITS)) return -2;
+    const int g = q_heads / kv_heads;
+    const int hpw = g < 4 ? g : 4, tbw = 4 / hpw;
+    if (group_tokens < 1 || group_tokens > 16 * tbw) return -3;
+    DiffArgs a{(const elem_t*)q, q_stride, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots, positions,
+               (const elem_t*)gate, gate_stride, (elem_t*)out, partial, max_blocks, q_heads, kv_heads, head_dim, value_dim,
+               page_size, split_keys, max_splits, scale, softcap, temp_coef, temp_every, lam, out_scale, eps,
+               group_row0, group_ntok, group_tokens};
+    const int nch = (head_dim + 31) / 32;
+    int err;
+    if (nch == 1) err = launch_tiles<1>(a, group_row0, group_ntok, groups, hpw, tbw, stream);
+    else if (nch == 2) err = launch_tiles<2>(a, group_row0, group_ntok, groups, hpw, tbw, stream);
+    else err = launch_tiles<4>(a, group_row0, group_ntok, groups, hpw, tbw, stream);
+    if (err != 0 || max_splits == 1) return err;
+    diff_attention_combine_kernel<<<dim3(groups * group_tokens, q_heads), 64, 0, stream>>>(a);
+    return (int)hipGetLastError();
+#else
+    return -10;
+#endif
 }
 
 }  // extern "C"

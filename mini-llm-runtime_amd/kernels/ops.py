@@ -830,7 +830,7 @@ class Kernels:
         _tensor(v_pages, "v_pages", self.dtype, ndim=4)
         pages = k_pages.shape[0]
         _need(tuple(k_pages.shape) == (pages, kv_heads, page_size, 2 * head_dim), "k_pages: [pages, kv_heads, page, 2 * head_dim]")
-        _need(tuple(v_pages.shape) == (pages, kv_heads, page_size, value_dim), "v_pages: [pages, kv_heads, page, value_dim]")
+        _need(tuple(v_pages.shape) == (pages, kv_heads, value_dim, page_size), "v_pages: [pages, kv_heads, value_dim, page]")
 
     @timed("rope_kv", _tensors_work())
     def diff_kv_write(self, k, v, k_pages, v_pages, block_table, slots, positions, kv_heads, head_dim, value_dim, page_size):
@@ -880,7 +880,57 @@ class Kernels:
                _p(positions), _p(gate), ctypes.c_long(gs), _p(out), _p(partial), _c_int(rows), _c_int(q_heads),
                _c_int(kv_heads), _c_int(head_dim), _c_int(value_dim), _c_int(page_size), _c_float(scale),
                _c_float(softcap or 0.0), _c_float(temp_coef), _c_float(temp_every), _c_float(lam), _c_float(out_scale),
-               _c_float(eps), _c_int(split_keys), _c_int(max_splits), _stream()), "diff_attention")
+               _c_float(eps), _c_int(split_keys), _c_int(max_splits), _ptr(0), _ptr(0), _c_int(0), _c_int(0), _stream()),
+            "diff_attention")
+
+    def diff_tiles_supported(self, q_heads, kv_heads, head_dim, value_dim, page_size, q_stride=0, gate_stride=0):
+        """Whether the matrix-core kernel takes these sizes: the bfloat16 engine, head sizes in multiples of 16 up to
+        128, pages in multiples of 8 tokens, operands aligned to its 16-byte accesses."""
+        return (self.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 128 and value_dim % 16 == 0
+                and value_dim <= 128 and page_size % 8 == 0 and q_heads % kv_heads == 0 and q_stride % 8 == 0
+                and gate_stride % 4 == 0)
+
+    @staticmethod
+    def diff_tiles_group_tokens(q_heads, kv_heads):
+        """Tokens of a prompt portion that one workgroup of the matrix-core kernel takes: its four wavefronts serve
+        16 tokens of one query head each, up to four heads of one kv head side by side."""
+        return 16 * (4 // min(4, q_heads // kv_heads))
+
+    @timed("attention")
+    def diff_attention_tiles(self, q, k_pages, v_pages, block_table, slots, positions, gate, out, partial, group_row0,
+                             group_ntok, groups, group_tokens, q_heads, kv_heads, head_dim, value_dim, page_size, scale, lam,
+                             out_scale, eps, softcap=None, temp_coef=0.0, temp_every=1.0, split_keys=0, max_splits=1):
+        """As `diff_attention` for the rows of `groups` groups of consecutive tokens of one request each (first row,
+        number of tokens: device int32 vectors; at most `group_tokens` tokens a group), on the matrix cores."""
+        rows = q.shape[0]
+        qs = self._columns(q, "q", self.dtype, rows, q_heads * 2 * head_dim)
+        gs = self._columns(gate, "gate", self.dtype, rows, q_heads * value_dim) if gate is not None else 0
+        _need(self.diff_tiles_supported(q_heads, kv_heads, head_dim, value_dim, page_size, qs, gs),
+              "diff_attention_tiles: sizes not taken (see diff_tiles_supported)")
+        _need(q.data_ptr() % 16 == 0 and (gate is None or gate.data_ptr() % 8 == 0), "diff_attention_tiles: unaligned operands")
+        self._check_diff_cache(k_pages, v_pages, kv_heads, head_dim, value_dim, page_size)
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _tensor(positions, "positions", torch.int32, (rows,))
+        _tensor(out, "out", self.dtype, (rows, q_heads * value_dim))
+        _tensor(group_row0, "group_row0", torch.int32, (groups,))
+        _tensor(group_ntok, "group_ntok", torch.int32, (groups,))
+        _need(1 <= group_tokens <= self.diff_tiles_group_tokens(q_heads, kv_heads), "diff_attention_tiles: group too large")
+        max_splits = max(1, max_splits)
+        if max_splits > 1:
+            _tensor(partial, "partial", torch.float32, ndim=1)
+            _need(partial.numel() >= self.diff_partial_numel(groups * group_tokens, q_heads, value_dim, max_splits),
+                  "diff_attention_tiles: partial too small")
+            _need(split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0 and max_splits <= MAX_KEY_SPLITS,
+                  "diff_attention_tiles: key ranges must be multiples of 64 keys, at most 1024 of them")
+        _need(kv_heads * 4 <= 65535 and max_splits <= 65535, "diff_attention_tiles: grid too large")
+        fn = self._lib("diff_attention").mlr_diff_attention_tiles
+        _ok(fn(_p(q), ctypes.c_long(qs), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
+               _p(positions), _p(gate), ctypes.c_long(gs), _p(out), _p(partial if max_splits > 1 else None), _p(group_row0),
+               _p(group_ntok), _c_int(groups), _c_int(group_tokens), _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim),
+               _c_int(value_dim), _c_int(page_size), _c_float(scale), _c_float(softcap or 0.0), _c_float(temp_coef),
+               _c_float(temp_every), _c_float(lam), _c_float(out_scale), _c_float(eps), _c_int(split_keys),
+               _c_int(max_splits), _stream()), "diff_attention_tiles")
 
     # -- sampling ----------------------------------------------------------------------------
     def sample_scratch(self, rows):

@@ -7,7 +7,11 @@ share a kv head.  There is no rotation: a query's position enters as a factor on
 (`QueryTemperature`), a score is squashed by `softcap * tanh(score / softcap)`, and position p sees keys 0..p.
 
 Per token the cache keeps the keys of both maps [kv_heads, 2 * head_dim] and the values [kv_heads, value_dim]
-(`PagedSpec`).  q, k, v and the gate are one stacked projection of the mixer's input."""
+(`PagedSpec`).  q, k, v and the gate are one stacked projection of the mixer's input.
+
+The float engine runs every token through the scalar kernel with key ranges of one width (the same bits however a
+request is cut or batched); the bfloat16 engine takes prompt portions and single tokens to the matrix-core kernel
+where it takes the sizes, a token's keys cut into ranges where the batch alone would not fill the GPU."""
 from __future__ import annotations
 
 import math
@@ -19,6 +23,7 @@ from ..weights.loader import WeightSpec, stacked
 from .registry import PartError, register_part
 
 PARTIAL_CAP = 32 << 20        # floats that the key ranges' partial results of one launch may take at most
+SMALL_GROUP = 4               # tokens: a request that brings more of them to a step is a prompt portion
 
 
 @register_part("mixer", "diff_attention")
@@ -37,6 +42,7 @@ class DiffAttention:
         self.v_width, self.o_width = s.kv_heads * s.value_dim, s.q_heads * s.value_dim
         self.proj = self.o = None
         self.lam = None
+        self._partial_floats = PARTIAL_CAP
 
     def weight_specs(self):
         s = self.spec
@@ -63,7 +69,8 @@ class DiffAttention:
 
     def cache_spec(self):
         s = self.spec
-        return PagedSpec((("k", (s.kv_heads, PAGE, 2 * s.head_dim)), ("v", (s.kv_heads, PAGE, s.value_dim))), None)
+        # (values transposed within a page: the keys of one channel side by side, as the matrix cores want them)
+        return PagedSpec((("k", (s.kv_heads, PAGE, 2 * s.head_dim)), ("v", (s.kv_heads, s.value_dim, PAGE))), None)
 
     def libraries(self):
         return ["gemm", "diff_attention"]
@@ -85,9 +92,52 @@ class DiffAttention:
         _, splits = self._splits(limits["max_length"], limits["split_keys"])
         per_row = Kernels.diff_partial_numel(1, s.q_heads, s.value_dim, splits)
         total = self.q_width + self.k_width + self.v_width + (self.o_width if s.gate is not None else 0)
-        return {("diff_proj", dtype): rows * total, ("attn", dtype): rows * self.o_width,
+        self._partial_floats = max(per_row, min(rows * per_row, PARTIAL_CAP))
+        plan = {("diff_proj", dtype): rows * total, ("attn", dtype): rows * self.o_width,
                 ("mixer_out", dtype): rows * s.hidden,
                 ("diff_partial", torch.float32): max(per_row, min(rows * per_row, PARTIAL_CAP))}
+        for factor in (4, 8, 16):
+            plan[(f"token_groups_{SMALL_GROUP}_{factor}", torch.int32)] = 2 * rows + 2
+        return plan
+
+    def _tile_splits(self, ctx, units, places, budget):
+        """(width of a key range, number of ranges) for a launch of the matrix-core kernel that has `units`
+        workgroups without ranges and `places` rows of partial results: no ranges where the batch fills the GPU or
+        the context is short; else the widest ranges that still give `target_workgroups`, widened further until
+        the partial results fit `budget` floats."""
+        s = self.spec
+        base, longest = ctx.split_keys, ctx.max_context
+        if base <= 0 or longest <= base or units >= ctx.target_workgroups:
+            return 0, 1
+        keys = base
+        while keys * 2 < longest and units * (-(-longest // (keys * 2))) >= ctx.target_workgroups:
+            keys *= 2
+        numel = lambda k: ctx.kernels.diff_partial_numel(places, s.q_heads, s.value_dim, -(-longest // k))
+        while (numel(keys) > budget or -(-longest // keys) > 1024) and keys < longest:
+            keys *= 2
+        splits = -(-longest // keys)
+        return (keys, splits) if splits > 1 else (0, 1)
+
+    def _attend_tiles(self, ctx, q, gate, view, attn):
+        """The bfloat16 engine on the matrix cores: prompt portions in groups of 16 to 64 tokens, single tokens and
+        portions of up to SMALL_GROUP tokens in groups of their own."""
+        s = self.spec
+        k = ctx.kernels
+        tokens = k.diff_tiles_group_tokens(s.q_heads, s.kv_heads)
+        small, big, _ = ctx.token_groups(SMALL_GROUP, tokens // SMALL_GROUP)
+        temp = s.q_temperature
+        g = s.q_heads // s.kv_heads
+        per_group = s.kv_heads * (-(-g // min(4, g)))
+        partial = ctx.workspace.get("diff_partial", (self._partial_floats,), torch.float32)
+        for (first, count, n), group_tokens in ((big, tokens), (small, SMALL_GROUP)):
+            if n == 0:
+                continue
+            split_keys, splits = self._tile_splits(ctx, n * per_group, n * group_tokens, partial.numel())
+            k.diff_attention_tiles(q, view.tensors["k"], view.tensors["v"], view.block_table, ctx.slots, ctx.positions, gate,
+                                   attn, partial, first, count, n, group_tokens, s.q_heads, s.kv_heads, s.head_dim,
+                                   s.value_dim, view.page_size, float(s.scale), self.lam, float(s.out_scale), float(s.eps),
+                                   softcap=s.softcap, temp_coef=temp.coef if temp else 0.0,
+                                   temp_every=temp.every if temp else 1.0, split_keys=split_keys, max_splits=splits)
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
@@ -106,6 +156,12 @@ class DiffAttention:
             k.diff_kv_write(keys, values, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, s.kv_heads,
                             s.head_dim, s.value_dim, view.page_size)
         attn = ctx.workspace.get("attn", (m, self.o_width), x.dtype)
+        if k.diff_tiles_supported(s.q_heads, s.kv_heads, s.head_dim, s.value_dim, view.page_size, proj.stride(0), proj.stride(0)) \
+                and a % 8 == 0 and c % 4 == 0:
+            self._attend_tiles(ctx, q, gate, view, attn)
+            out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
+            k.gemm(attn, self.o, out)
+            return out
         split_keys, splits = self._splits(ctx.max_context, ctx.split_keys)
         per_row = k.diff_partial_numel(1, s.q_heads, s.value_dim, splits)
         chunk = max(1, min(m, PARTIAL_CAP // per_row))

@@ -220,7 +220,7 @@ def paged(k, dtype, keys, values, heads_kv, dim, vdim, page, order):
     n = keys.shape[0]
     blocks = -(-n // page)
     k_pages = torch.full((len(order) + 1, heads_kv, page, 2 * dim), float("nan"), dtype=dtype, device="cuda")
-    v_pages = torch.full((len(order) + 1, heads_kv, page, vdim), float("nan"), dtype=dtype, device="cuda")
+    v_pages = torch.full((len(order) + 1, heads_kv, vdim, page), float("nan"), dtype=dtype, device="cuda")
     table = torch.full((3, blocks + 2), -1, dtype=torch.int32, device="cuda")
     table[1, :blocks] = torch.tensor(order[:blocks], dtype=torch.int32)
     slots = torch.ones(n, dtype=torch.int32, device="cuda")
@@ -229,9 +229,38 @@ def paged(k, dtype, keys, values, heads_kv, dim, vdim, page, order):
     return k_pages, v_pages, table, slots, pos
 
 
-@pytest.mark.parametrize("dtype_name", DTYPES)
+def attend(k, path, q, pages, gate, heads, kv, dim, vdim, page, split_keys, constants, **more):
+    """The scalar kernel over all rows, or the matrix-core kernel over the rows cut into groups: portions of the
+    kernel's own size, then a ragged end of groups of up to four tokens (as the mixer forms them)."""
+    k_pages, v_pages, table, slots, pos = pages
+    n = q.shape[0]
+    splits = 1 if split_keys == 0 else -(-n // split_keys)
+    out = torch.full((n, heads * vdim), float("nan"), dtype=q.dtype, device="cuda")
+    if path == "scalar":
+        partial = torch.empty(k.diff_partial_numel(n, heads, vdim, splits), device="cuda")
+        k.diff_attention(q, k_pages, v_pages, table, slots, pos, gate, out, partial, heads, kv, dim, vdim, page, *constants,
+                         split_keys=split_keys, max_splits=splits, **more)
+        return out
+    tokens = k.diff_tiles_group_tokens(heads, kv)
+    tail = min(n, 7)
+    big = list(range(0, n - tail, tokens))
+    ints = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    for first, count, size in ((big, [min(tokens, n - tail - f) for f in big], tokens),
+                               ([n - tail, n - tail + 4][:1 + (tail > 4)], [min(4, tail), tail - 4][:1 + (tail > 4)], 4)):
+        if not first:
+            continue
+        partial = torch.empty(k.diff_partial_numel(len(first) * size, heads, vdim, splits), device="cuda")
+        k.diff_attention_tiles(q, k_pages, v_pages, table, slots, pos, gate, out, partial, ints(first), ints(count), len(first),
+                               size, heads, kv, dim, vdim, page, *constants, split_keys=split_keys, max_splits=splits, **more)
+    return out
+
+
+PATHS = [("float32", "scalar"), ("bfloat16", "scalar"), ("bfloat16", "tiles")]
+
+
+@pytest.mark.parametrize("dtype_name,path", PATHS)
 @pytest.mark.parametrize("split_keys", [0, 64, 128])
-def test_differential_attention_finds_one_key_wherever_it_lies(dtype_name, split_keys):
+def test_differential_attention_finds_one_key_wherever_it_lies(dtype_name, path, split_keys):
     """One query head, 700 tokens; the query of the last token is made to match the key at ONE position on map 1
     (and the key next to it on map 2) so strongly that the softmax holds nothing else: the output is then the
     normed difference of two known values.  The position is moved over the first tokens, page and key-range
@@ -240,7 +269,7 @@ def test_differential_attention_finds_one_key_wherever_it_lies(dtype_name, split
     dtype = DTYPES[dtype_name]
     k = Kernels(dtype)
     rng = np.random.default_rng(5)
-    n, dim, vdim, page = 700, 24, 40, 8
+    n, dim, vdim, page = 700, 32, 48, 8
     keys = rng.normal(size=(n, 2 * dim)) * 0.05
     values = rng.normal(size=(n, vdim))
     order = list(rng.permutation(n // page + 2))
@@ -255,12 +284,8 @@ def test_differential_attention_finds_one_key_wherever_it_lies(dtype_name, split
         q[-1, :dim], q[-1, dim:] = 8.0 * direction, -8.0 * direction
         gate = rng.normal(size=(n, vdim))
         kq, kk, kv, kg = (rounded(x, dtype) for x in (q, kt, values, gate))
-        k_pages, v_pages, table, slots, pos = paged(k, dtype, kk, kv, 1, dim, vdim, page, order)
-        splits = 1 if split_keys == 0 else -(-n // split_keys)
-        out = torch.empty(n, vdim, dtype=dtype, device="cuda")
-        partial = torch.empty(k.diff_partial_numel(n, 1, vdim, splits), device="cuda")
-        k.diff_attention(kq, k_pages, v_pages, table, slots, pos, kg, out, partial, 1, 1, dim, vdim, page, 1.0, 0.5, 0.7, 1e-6,
-                         softcap=None, temp_coef=0.0, split_keys=split_keys, max_splits=splits)
+        out = attend(k, path, kq, paged(k, dtype, kk, kv, 1, dim, vdim, page, order), kg, 1, 1, dim, vdim, page, split_keys,
+                     (1.0, 0.5, 0.7, 1e-6), softcap=None, temp_coef=0.0)
         v = kv.double().cpu().numpy()
         o = v[target] - 0.5 * v[other]               # scores of 32 against at most 2: every other weight is < 1e-12
         want = o / np.sqrt((o * o).mean() + 1e-6) * 0.7 * P.sigmoid(kg.double().cpu().numpy()[-1])
@@ -268,24 +293,23 @@ def test_differential_attention_finds_one_key_wherever_it_lies(dtype_name, split
         np.testing.assert_allclose(out[-1].double().cpu().numpy(), want, atol=tol * np.abs(want).max(), rtol=tol, err_msg=str(target))
 
 
-@pytest.mark.parametrize("dtype_name", DTYPES)
-def test_differential_attention_against_the_plain_maps(dtype_name):
-    """Three query heads on three kv heads and four on two, with the cap, the query's factor and the gate."""
+@pytest.mark.parametrize("dtype_name,path", PATHS)
+def test_differential_attention_against_the_plain_maps(dtype_name, path):
+    """Query heads that share kv heads or do not, with the cap, the query's factor and the gate."""
     from mini_llm_runtime_amd.kernels import Kernels
     dtype = DTYPES[dtype_name]
     k = Kernels(dtype)
     rng = np.random.default_rng(8)
-    for heads, kv, dim, vdim, page in ((3, 3, 20, 72, 4), (4, 2, 16, 32, 16), (2, 1, 130, 200, 8)):
+    sizes = ((3, 3, 20, 72, 4), (4, 2, 16, 32, 16), (2, 1, 130, 200, 8)) if path == "scalar" else \
+        ((3, 3, 16, 80, 8), (4, 2, 16, 32, 16), (8, 1, 48, 16, 8), (6, 2, 128, 128, 32), (1, 1, 64, 96, 8))
+    for heads, kv, dim, vdim, page in sizes:
         n = 150
         q, keys = rng.normal(size=(n, heads * 2 * dim)), rng.normal(size=(n, kv * 2 * dim))
         values, gate = rng.normal(size=(n, kv * vdim)), rng.normal(size=(n, heads * vdim))
         kq, kk, kv_t, kg = (rounded(x, dtype) for x in (q, keys, values, gate))
-        k_pages, v_pages, table, slots, pos = paged(k, dtype, kk, kv_t, kv, dim, vdim, page, list(rng.permutation(n // page + 2)))
-        out = torch.empty(n, heads * vdim, dtype=dtype, device="cuda")
-        splits = -(-n // 64)
-        partial = torch.empty(k.diff_partial_numel(n, heads, vdim, splits), device="cuda")
-        k.diff_attention(kq, k_pages, v_pages, table, slots, pos, kg, out, partial, heads, kv, dim, vdim, page, 0.3, 0.45, 0.8, 1e-5,
-                         softcap=2.5, temp_coef=0.7, temp_every=9.0, split_keys=64, max_splits=splits)
+        pages = paged(k, dtype, kk, kv_t, kv, dim, vdim, page, list(rng.permutation(n // page + 2)))
+        out = attend(k, path, kq, pages, kg, heads, kv, dim, vdim, page, 64 if heads != 3 else 0, (0.3, 0.45, 0.8, 1e-5),
+                     softcap=2.5, temp_coef=0.7, temp_every=9.0)
         q, keys, values, gate = (t.double().cpu().numpy() for t in (kq, kk, kv_t, kg))
         q = q.reshape(n, heads, 2, dim) * P.query_temperature(np.arange(n), 0.7, 9.0)[:, None, None, None]
         keys, values = keys.reshape(n, kv, 2, dim), values.reshape(n, kv, vdim)
