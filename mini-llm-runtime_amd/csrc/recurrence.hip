@@ -7,6 +7,12 @@
 // state that the step leads to is written to `stage + slot * stride` (the engine makes it live when every
 // layer has run).  Every sum is taken in an order that depends on the token's own data only, so a token's
 // result does not depend on how its request was cut into steps or on what else the batch holds.
+//
+// Long portions (the bfloat16 engine) run the recurrence over pieces of a request side by side, in three passes:
+// every piece from a zero state, leaving its last state L_c and the product A_c of its decays; then, piece after
+// piece, the state each piece starts from, S_(c+1) = diag(A_c) S_c + L_c (element by element, from the live
+// state); then every piece again from its S_c, writing the outputs.  Twice the arithmetic, as many workgroups as
+// pieces; the result differs from the token-by-token order by 32-bit rounding only.
 #include "common.h"
 
 __device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
@@ -96,6 +102,8 @@ struct ScanArgs {
     const int32_t* seg_first; const int32_t* seg_count; const int32_t* slots;
     int heads, heads_per_group, N, V, decay_per_channel, write_state;
     float q_scale;
+    float* piece_state;                        // [pieces][heads][N][V]: L_c after the first pass, S_c after the second
+    float* piece_decay;                        // [pieces][heads][N]: A_c
 };
 
 #define SCAN_COLS 64
@@ -105,7 +113,10 @@ struct ScanArgs {
 // of S for its 64 columns in registers, a lane a column.  Tokens are staged TILE at a time through LDS
 // (decays exponentiated, q scaled, v scaled); after a tile the four partial sums of o are added in the order
 // of the parts.
-template <int NR, int TILE>
+// MODE 0: a request's rows of the step from its live state to the staged one.  MODE 1: a piece from a zero state,
+// no outputs; leaves L_c and A_c.  MODE 2: a piece from S_c, outputs only.  (In modes 1 and 2 `seg_first` and
+// `seg_count` name the pieces.)
+template <int NR, int TILE, int MODE>
 __global__ __launch_bounds__(256) void linear_recurrence_kernel(ScanArgs a) {
     constexpr int NPAD = NR * SCAN_PARTS;
     extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -122,11 +133,14 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(ScanArgs a) {
     const int N = a.N, V = a.V;
     const int qk_head = head / a.heads_per_group;
     const size_t state_at = (size_t)slot * a.state_stride + (size_t)head * N * V;
-    float S[NR];
+    const size_t piece_at = ((size_t)seg * a.heads + head) * N * V;
+    float S[NR], A[NR];
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
         const int i = part * NR + r;
-        S[r] = (i < N && col < V) ? a.live[state_at + (size_t)i * V + col] : 0.f;
+        const bool in = i < N && col < V;
+        S[r] = MODE == 1 || !in ? 0.f : MODE == 0 ? a.live[state_at + (size_t)i * V + col] : a.piece_state[piece_at + (size_t)i * V + col];
+        A[r] = 1.f;
     }
     for (int t0 = 0; t0 < n; t0 += TILE) {
         const int nt = min(TILE, n - t0);
@@ -162,10 +176,12 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(ScanArgs a) {
 #pragma unroll
             for (int r = 0; r < NR; ++r) {
                 S[r] = at[r] * S[r] + kt[r] * x;
-                o += qt[r] * S[r];
+                if (MODE == 1) A[r] *= at[r];
+                else o += qt[r] * S[r];
             }
-            o_lds[(part * TILE + t) * SCAN_COLS + j] = o;
+            if (MODE != 1) o_lds[(part * TILE + t) * SCAN_COLS + j] = o;
         }
+        if (MODE == 1) continue;
         __syncthreads();
         for (int idx = threadIdx.x; idx < nt * SCAN_COLS; idx += 256) {
             const int t = idx / SCAN_COLS, c = col0 + idx % SCAN_COLS;
@@ -178,12 +194,39 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(ScanArgs a) {
             a.out[row * ((size_t)a.heads * V) + head * V + c] = o;
         }
     }
-    if (a.write_state && col < V) {
+    if (MODE == 0 && a.write_state && col < V) {
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
             const int i = part * NR + r;
             if (i < N) a.stage[state_at + (size_t)i * V + col] = S[r];
         }
+    }
+    if (MODE == 1) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int i = part * NR + r;
+            if (i < N && col < V) a.piece_state[piece_at + (size_t)i * V + col] = S[r];
+            if (i < N && col == 0) a.piece_decay[((size_t)seg * a.heads + head) * N + i] = A[r];
+        }
+    }
+}
+
+// The second pass: one thread per element (head, i, j) of the state walks the pieces in their order.  A piece
+// whose request differs from the piece before starts from that request's live state; where a request's pieces
+// end its state is staged.  piece_state[c] holds L_c on entry and S_c, the state piece c starts from, on exit.
+__global__ void piece_states_kernel(ScanArgs a, int pieces) {
+    const size_t per = (size_t)a.heads * a.N * a.V;
+    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= per) return;
+    const size_t hi = e / a.V;                 // head * N + i
+    float S = 0.f;
+    for (int c = 0; c < pieces; ++c) {
+        const int slot = a.slots[a.seg_first[c]];
+        if (c == 0 || a.slots[a.seg_first[c - 1]] != slot) S = a.live[(size_t)slot * a.state_stride + e];
+        const float last = a.piece_state[(size_t)c * per + e];
+        a.piece_state[(size_t)c * per + e] = S;
+        S = a.piece_decay[(size_t)c * a.heads * a.N + hi] * S + last;
+        if (a.write_state && (c + 1 == pieces || a.slots[a.seg_first[c + 1]] != slot)) a.stage[(size_t)slot * a.state_stride + e] = S;
     }
 }
 
@@ -191,7 +234,18 @@ template <int NR, int TILE>
 static int launch_scan(const ScanArgs& a, int segments, hipStream_t stream) {
     const size_t lds = sizeof(float) * ((size_t)3 * TILE * NR * SCAN_PARTS + (size_t)TILE * SCAN_COLS * (1 + SCAN_PARTS));
     dim3 grid(segments, a.heads, (a.V + SCAN_COLS - 1) / SCAN_COLS);
-    linear_recurrence_kernel<NR, TILE><<<grid, 256, lds, stream>>>(a);
+    if (a.piece_state == nullptr) {
+        linear_recurrence_kernel<NR, TILE, 0><<<grid, 256, lds, stream>>>(a);
+        return (int)hipGetLastError();
+    }
+    linear_recurrence_kernel<NR, TILE, 1><<<grid, 256, lds, stream>>>(a);
+    int err = (int)hipGetLastError();
+    if (err != 0) return err;
+    const size_t per = (size_t)a.heads * a.N * a.V;
+    piece_states_kernel<<<(unsigned)((per + 255) / 256), 256, 0, stream>>>(a, segments);
+    err = (int)hipGetLastError();
+    if (err != 0) return err;
+    linear_recurrence_kernel<NR, TILE, 2><<<grid, 256, lds, stream>>>(a);
     return (int)hipGetLastError();
 }
 
@@ -233,12 +287,15 @@ int mlr_linear_recurrence(const void* q, long q_stride, const void* k, long k_st
                           long v_scale_stride, const float* skip, float q_scale, float* out, const float* live, float* stage,
                           long state_stride, const int32_t* seg_first, const int32_t* seg_count, const int32_t* slots,
                           int segments, int heads, int heads_per_group, int n_keys, int n_values, int write_state,
-                          hipStream_t stream) {
+                          float* piece_state, float* piece_decay, hipStream_t stream) {
+    // piece_state, piece_decay given: `seg_first`/`seg_count` name pieces of requests (a request's pieces one after
+    // the other), run side by side in three passes; [segments][heads][n_keys][n_values] and [segments][heads][n_keys]
     if (segments <= 0) return 0;
     if (n_keys < 1 || n_keys > 256 || n_values < 1 || heads < 1 || heads_per_group < 1 || heads % heads_per_group) return -1;
     ScanArgs a{(const elem_t*)q, q_stride, (const elem_t*)k, k_stride, (const elem_t*)v, v_stride, log_decay, decay_stride,
                v_scale, v_scale_stride, skip, out, live, stage, state_stride, seg_first, seg_count, slots, heads,
-               heads_per_group, n_keys, n_values, decay_per_channel, write_state, q_scale};
+               heads_per_group, n_keys, n_values, decay_per_channel, write_state, q_scale, piece_state, piece_decay};
+    if ((piece_state == nullptr) != (piece_decay == nullptr)) return -2;
     const int nr = (n_keys + SCAN_PARTS - 1) / SCAN_PARTS;
     if (nr <= 8) return launch_scan<8, 16>(a, segments, stream);
     if (nr <= 16) return launch_scan<16, 16>(a, segments, stream);

@@ -784,12 +784,15 @@ class Kernels:
     @timed("recurrence", _tensors_work())
     def linear_recurrence(self, q, k, v, log_decay, out, live, stage, state_offset, seg_first, seg_count, segments, slots,
                           heads, n_keys, n_values, heads_per_group=1, v_scale=None, skip=None, q_scale=1.0,
-                          write_state=True):
+                          write_state=True, piece_state=None, piece_decay=None):
         """Per request of the step and head, from the live state: S_t = diag(exp(log_decay_t)) S_(t-1) + k_t (v_scale_t
         v_t)^T, out_t = S_t^T (q_scale q_t) + skip[head] v_t.  q, k: columns [rows, (heads / heads_per_group) * n_keys];
         v: columns [rows, heads * n_values]; log_decay float [rows, heads * n_keys] (a decay per key channel) or
         [rows, heads] (one per head); v_scale float [rows, heads]; the state [heads][n_keys][n_values] floats from
-        `state_offset` on in a slot's row of `live`/`stage`."""
+        `state_offset` on in a slot's row of `live`/`stage`.
+        With `piece_state` float [segments * heads * n_keys * n_values] and `piece_decay` float [segments * heads *
+        n_keys]: `seg_first`/`seg_count` name PIECES of requests (a request's pieces one after the other), which run
+        side by side in three passes; the result differs from the token-by-token order by 32-bit rounding."""
         rows = v.shape[0]
         groups = heads // heads_per_group
         _need(heads >= 1 and heads_per_group >= 1 and heads % heads_per_group == 0, "linear_recurrence: heads and groups")
@@ -812,6 +815,12 @@ class Kernels:
         _tensor(seg_count, "seg_count", torch.int32, (segments,))
         _tensor(slots, "slots", torch.int32, (rows,))
         _need(segments <= 65535 * 32 and heads <= 65535, "linear_recurrence: too many requests or heads for the grid")
+        _need((piece_state is None) == (piece_decay is None), "linear_recurrence: piece_state and piece_decay go together")
+        if piece_state is not None:
+            _tensor(piece_state, "piece_state", torch.float32, ndim=1)
+            _tensor(piece_decay, "piece_decay", torch.float32, ndim=1)
+            _need(piece_state.numel() >= segments * heads * n_keys * n_values and piece_decay.numel() >= segments * heads * n_keys,
+                  "linear_recurrence: the pieces' buffers are too small")
         fn = self._lib("recurrence").mlr_linear_recurrence
         at = state_offset * 4
         _ok(fn(_p(q), ctypes.c_long(qs), _p(k), ctypes.c_long(ks), _p(v), ctypes.c_long(vs), _p(log_decay),
@@ -819,7 +828,8 @@ class Kernels:
                ctypes.c_long(heads if v_scale is not None else 0), _p(skip), _c_float(q_scale), _p(out),
                _ptr(live.data_ptr() + at), _ptr(stage.data_ptr() + at), ctypes.c_long(live.stride(0)), _p(seg_first),
                _p(seg_count), _p(slots), _c_int(segments), _c_int(heads), _c_int(heads_per_group), _c_int(n_keys),
-               _c_int(n_values), _c_int(1 if write_state else 0), _stream()), "linear_recurrence")
+               _c_int(n_values), _c_int(1 if write_state else 0), _p(piece_state), _p(piece_decay), _stream()),
+            "linear_recurrence")
 
     # -- differential attention -----------------------------------------------------------------------
     DIFF_MAX_HEAD_DIM = 256

@@ -14,12 +14,41 @@ from ..weights.loader import WeightSpec, stacked
 from .registry import PartError, register_part
 
 WHOLE = 1 << 30          # `StepContext.token_groups(WHOLE)`: every request of the step as one group of rows
+PIECE = 128              # tokens of a piece when a step's portions run in pieces side by side
+PIECES_FROM = 512        # rows of a step from which they do (the bfloat16 engine)
+PIECE_FLOATS = 64 << 20  # floats that the pieces' states may take; a step with more runs token by token
 
 
 def _requests(ctx):
     """(first row, number of rows, how many) of the step's requests, as device vectors."""
     (first, count, n), _, _ = ctx.token_groups(WHOLE, 0)
     return first, count, n
+
+
+def _recurrence(ctx, state_floats, heads, n_keys, *args, **kwargs):
+    """`Kernels.linear_recurrence` over the step's requests: token by token (the float engine always: the same bits
+    however a request is cut), or, for the many rows of prompt portions in the bfloat16 engine, in pieces of PIECE
+    tokens side by side."""
+    rows = ctx.n_tokens
+    pieces_most = rows // PIECE + len(ctx.segments)
+    if ctx.dtype == torch.bfloat16 and rows >= PIECES_FROM and pieces_most * state_floats <= PIECE_FLOATS:
+        (first, count, n), _, _ = ctx.token_groups(PIECE, 0)
+        kwargs["piece_state"] = ctx.workspace.get("recurrent_pieces", (n * state_floats,), torch.float32)
+        kwargs["piece_decay"] = ctx.workspace.get("recurrent_piece_decay", (n * heads * n_keys,), torch.float32)
+    else:
+        first, count, n = _requests(ctx)
+    ctx.kernels.linear_recurrence(*args[:8], first, count, n, *args[8:], **kwargs)
+
+
+def _pieces_plan(rows, state_floats, heads, n_keys):
+    """Scratch buffers of `_recurrence` for a step of at most `rows` tokens (every request may add a ragged piece;
+    at most `rows` requests, but then there are no pieces: bounded by the rows a step with pieces has)."""
+    if rows < PIECES_FROM:
+        return {}
+    pieces = min(2 * (rows // PIECE) + 1, max(1, PIECE_FLOATS // state_floats))
+    return {("recurrent_pieces", torch.float32): pieces * state_floats,
+            ("recurrent_piece_decay", torch.float32): pieces * heads * n_keys,
+            (f"token_groups_{PIECE}_0", torch.int32): 2 * rows + 2}
 
 
 @register_part("mixer", "gla")
@@ -68,7 +97,8 @@ class GatedLinearAttention:
         return {("gla_proj", dtype): rows * (2 * self.qk_width + 2 * self.v_width), ("gla_low", dtype): rows * rank,
                 ("gla_z", dtype): rows * self.qk_width, ("log_decay", torch.float32): rows * self.qk_width,
                 ("recurrent_out", torch.float32): rows * self.v_width, ("recurrent_normed", dtype): rows * self.v_width,
-                ("mixer_out", dtype): rows * s.hidden, (f"token_groups_{WHOLE}_0", torch.int32): 2 * rows + 2}
+                ("mixer_out", dtype): rows * s.hidden, (f"token_groups_{WHOLE}_0", torch.int32): 2 * rows + 2,
+                **_pieces_plan(rows, s.heads * s.head_dim * s.value_dim, s.heads, s.head_dim)}
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
@@ -85,11 +115,11 @@ class GatedLinearAttention:
         k.gla_log_decay(z, self.a2_bias, log_decay, float(s.tau))
         a, b = self.qk_width, 2 * self.qk_width
         c = b + self.v_width
-        first, count, n = _requests(ctx)
         o = ws.get("recurrent_out", (m, self.v_width), torch.float32)
-        k.linear_recurrence(proj[:, :a], proj[:, a:b], proj[:, b:c], log_decay, o, ctx.cache.state_view(cache_id),
-                            ctx.cache.state_stage(cache_id), 0, first, count, n, ctx.slots, s.heads, s.head_dim,
-                            s.value_dim, q_scale=float(s.head_dim) ** -0.5, write_state=write_cache)
+        _recurrence(ctx, s.heads * s.head_dim * s.value_dim, s.heads, s.head_dim,
+                    proj[:, :a], proj[:, a:b], proj[:, b:c], log_decay, o, ctx.cache.state_view(cache_id),
+                    ctx.cache.state_stage(cache_id), 0, ctx.slots, s.heads, s.head_dim,
+                    s.value_dim, q_scale=float(s.head_dim) ** -0.5, write_state=write_cache)
         y = ws.get("recurrent_normed", (m, self.v_width), x.dtype)
         k.gated_part_norm(o, proj[:, c:], self.norm, y, s.value_dim, float(s.eps), gate_first=False, gate_kind="silu")
         out = ws.get("mixer_out", (m, s.hidden), x.dtype)
@@ -148,7 +178,8 @@ class Mamba2:
         return {("mamba_proj", dtype): rows * (2 * self.inner + 2 * self.bc + s.heads), ("mamba_conv", dtype): rows * self.channels,
                 ("mamba_dt", torch.float32): rows * s.heads, ("log_decay", torch.float32): rows * s.heads,
                 ("recurrent_out", torch.float32): rows * self.inner, ("recurrent_normed", dtype): rows * self.inner,
-                ("mixer_out", dtype): rows * s.hidden, (f"token_groups_{WHOLE}_0", torch.int32): 2 * rows + 2}
+                ("mixer_out", dtype): rows * s.hidden, (f"token_groups_{WHOLE}_0", torch.int32): 2 * rows + 2,
+                **_pieces_plan(rows, self.state_floats, s.heads, s.state)}
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
@@ -166,11 +197,11 @@ class Mamba2:
         dt = ws.get("mamba_dt", (m, s.heads), torch.float32)
         log_decay = ws.get("log_decay", (m, s.heads), torch.float32)
         k.mamba_step(raw, self.dt_bias, self.a_log, dt, log_decay)
-        first, count, n = _requests(ctx)
         y = ws.get("recurrent_out", (m, inner), torch.float32)
-        k.linear_recurrence(conv[:, inner + bc:], conv[:, inner:inner + bc], conv[:, :inner], log_decay, y, live, stage, 0,
-                            first, count, n, ctx.slots, s.heads, s.state, s.value_dim, heads_per_group=s.heads // s.groups,
-                            v_scale=dt, skip=self.skip, write_state=write_cache)
+        _recurrence(ctx, self.state_floats, s.heads, s.state,
+                    conv[:, inner + bc:], conv[:, inner:inner + bc], conv[:, :inner], log_decay, y, live, stage, 0,
+                    ctx.slots, s.heads, s.state, s.value_dim, heads_per_group=s.heads // s.groups,
+                    v_scale=dt, skip=self.skip, write_state=write_cache)
         normed = ws.get("recurrent_normed", (m, inner), x.dtype)
         k.gated_part_norm(y, z, self.norm, normed, inner // s.norm_groups, float(s.eps), gate_first=True, gate_kind="silu")
         out = ws.get("mixer_out", (m, s.hidden), x.dtype)

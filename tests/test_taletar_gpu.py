@@ -83,10 +83,11 @@ def load(folders, name, dtype_name):
 def runner_for(model, max_tokens, **kwargs):
     from mini_llm_runtime_amd.engine import Runner
     kwargs.setdefault("split_keys", 64)            # (key ranges of 64: prompts of 150 tokens cross two borders)
-    return Runner(model, max_tokens=max_tokens, max_slots=4, page_size=8, max_length=512, **kwargs)
+    kwargs.setdefault("max_length", 512)
+    return Runner(model, max_tokens=max_tokens, max_slots=4, page_size=8, **kwargs)
 
 
-def close(got, want, dtype_name, scale):
+def close(got, want, dtype_name, scale, outliers=None):
     """Rows against float64: the float engine to rounding at every row; the bfloat16 engine to 4 % of the largest
     logit at the worst place and 1.2 % in the root mean square, where one row in fifty may reach three times that
     (a head's output is normed: a token whose head output is nearly zero, the first of a sequence for one, is
@@ -101,7 +102,7 @@ def close(got, want, dtype_name, scale):
         elif not (err.max() <= 0.04 * scale and np.sqrt((err ** 2).mean()) <= 0.012 * scale):
             assert err.max() <= 0.12 * scale and np.sqrt((err ** 2).mean()) <= 0.036 * scale, (key, err.max(), scale)
             over.append(key)
-    assert len(over) <= max(1, len(want) // 50), over
+    assert len(over) <= (max(1, len(want) // 50) if outliers is None else outliers), over
 
 
 def idle(r):
@@ -178,6 +179,56 @@ def test_linear_recurrence_carries_its_state_across_steps(dtype_name, heads, per
     for s in lengths:
         scale = np.abs(want[s]).max()
         np.testing.assert_allclose(np.concatenate(got[s]), want[s], atol=2e-5 * scale, rtol=2e-5)
+
+
+@pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("heads,per_group,keys,values,per_channel", [(2, 1, 24, 40, True), (4, 2, 16, 70, False)])
+def test_linear_recurrence_in_pieces_side_by_side(dtype_name, heads, per_group, keys, values, per_channel):
+    """Two requests, one of 300 tokens from a state that is not zero, cut into pieces of 64 tokens that run side by
+    side: outputs and the staged states against the token-by-token recurrence."""
+    from mini_llm_runtime_amd.kernels import Kernels
+    dtype = DTYPES[dtype_name]
+    k = Kernels(dtype)
+    rng = np.random.default_rng(11)
+    groups = heads // per_group
+    lengths, slot_of = [300, 5], [2, 0]
+    n = sum(lengths)
+    q, kk = rounded(rng.normal(size=(n, groups * keys)), dtype), rounded(rng.normal(size=(n, groups * keys)), dtype)
+    v = rounded(rng.normal(size=(n, heads * values)), dtype)
+    decay = torch.from_numpy(rng.uniform(-0.3, -0.001, size=(n, heads * (keys if per_channel else 1)))).float().cuda()
+    state = heads * keys * values
+    live = torch.from_numpy(rng.normal(size=(3, state))).float().cuda()
+    stage = torch.zeros_like(live)
+    first, count, slots = [], [], []
+    at = 0
+    for length, slot in zip(lengths, slot_of):
+        for a in range(0, length, 64):
+            first.append(at + a)
+            count.append(min(64, length - a))
+        slots += [slot] * length
+        at += length
+    ints = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    out = torch.full((n, heads * values), float("nan"), device="cuda")
+    pieces = len(first)
+    k.linear_recurrence(q, kk, v, decay, out, live, stage, 0, ints(first), ints(count), pieces, ints(slots), heads, keys, values,
+                        heads_per_group=per_group, piece_state=torch.empty(pieces * state, device="cuda"),
+                        piece_decay=torch.empty(pieces * heads * keys, device="cuda"))
+    q64, k64, v64, d64 = (t.double().cpu().numpy() for t in (q, kk, v, decay))
+    at = 0
+    for length, slot in zip(lengths, slot_of):
+        rows = slice(at, at + length)
+        for h in range(heads):
+            g = h // per_group
+            a = np.exp(d64[rows, h * keys:(h + 1) * keys]) if per_channel else np.repeat(np.exp(d64[rows, h:h + 1]), keys, axis=1)
+            s0 = live[slot].double().cpu().numpy()[h * keys * values:(h + 1) * keys * values].reshape(keys, values)
+            o, last = P.linear_recurrence(q64[rows, g * keys:(g + 1) * keys], k64[rows, g * keys:(g + 1) * keys],
+                                          v64[rows, h * values:(h + 1) * values], a, s0)
+            scale = np.abs(o).max()
+            np.testing.assert_allclose(out[rows, h * values:(h + 1) * values].double().cpu().numpy(), o, atol=3e-5 * scale, rtol=3e-5)
+            got = stage[slot].double().cpu().numpy()[h * keys * values:(h + 1) * keys * values].reshape(keys, values)
+            np.testing.assert_allclose(got, last, atol=3e-5 * np.abs(last).max(), rtol=3e-5)
+        at += length
+    assert torch.equal(stage[1], torch.zeros_like(stage[1]))
 
 
 @pytest.mark.parametrize("dtype_name", DTYPES)
@@ -438,6 +489,42 @@ def test_long_decoding_and_the_first_tokens(folders, name, dtype_name):
     r = runner_for(model, max_tokens=256, use_graphs=False)
     close(run_steps(r, last_one_by_one(reqs, tail=225)), want, dtype_name, scale)
     close(run_steps(r, portions(reqs, sizes=(1, 1, 2, 1, 3, 2))), {k: v for k, v in want.items()}, dtype_name, scale)
+    idle(r)
+
+
+@pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("name", ["mix", "odd"])
+def test_a_long_prompt_whole_in_portions_and_beside_single_tokens(folders, name, dtype_name):
+    """700 tokens: the bfloat16 engine runs the recurrent layers of so many rows in pieces side by side, and the
+    attention of the last portions walks several key ranges."""
+    from mini_llm_runtime_amd.engine import Entry
+    model_plain, _, _ = plain(folders, name)
+    model = load(folders, name, dtype_name)
+    reqs = make_requests(CONFIGS[name]["vocab"], [700, 30], seed=31)
+    long, short = reqs["r0"], reqs["r1"]
+    want_long, want_short = model_plain.logits(long), model_plain.logits(short)
+    scale = max(np.abs(want_long).max(), np.abs(want_short).max())
+    r = runner_for(model, max_tokens=1024, max_length=1024)
+    wanted = list(range(0, 700, 7)) + [699]
+
+    def check(rows, want, places):
+        # (the short request has two places, 22 and 24, that bfloat16 moves by 4 to 6 % of the largest logit also when it
+        # runs alone and whole: allowed here, bounded by three times the usual limit)
+        close({i: row for i, row in enumerate(rows.double().cpu().numpy())}, {i: want[p] for i, p in enumerate(places)}, dtype_name,
+              scale, outliers=2)
+    a = r.open_request()
+    check(r.step([Entry(a, long, wanted)]), want_long, wanted)
+    r.close_request(a)
+    a, b = r.open_request(), r.open_request()
+    r.step([Entry(b, short[:20], [])])
+    got = r.step([Entry(b, short[20:21], [0]), Entry(a, long[:600], wanted[:86])])       # a decoded token beside 600 tokens
+    check(got[:1], want_short, [20])
+    check(got[1:], want_long, wanted[:86])
+    got = r.step([Entry(a, long[600:], [w - 600 for w in wanted[86:]]), Entry(b, short[21:], list(range(9)))])
+    check(got[:len(wanted) - 86], want_long, wanted[86:])
+    check(got[len(wanted) - 86:], want_short, list(range(21, 30)))
+    r.close_request(a)
+    r.close_request(b)
     idle(r)
 
 
