@@ -238,21 +238,20 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 #define TKEYS 32
+#define TILES_PAGE_CACHE 2048    // page ids of a workgroup's key range kept in LDS: the host keeps a range within them
 
 // NCH: ceil(head_dim / 32) chunks of 32 channels a map; NDB: blocks of 16 value channels (value_dim <= 16 NDB).
 // head_dim and value_dim multiples of 16, the page size a multiple of 8.
 template <int NCH, int NDB>
-__global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffArgs a, const int32_t* __restrict__ group_row0,
-                                                                   const int32_t* __restrict__ group_ntok,
-                                                                   int heads_per_wg, int token_blocks) {
+__device__ __forceinline__ void diff_tiles_group(const DiffArgs& a, const int32_t* __restrict__ group_row0,
+                                                 const int32_t* __restrict__ group_ntok, int heads_per_wg, int token_blocks,
+                                                 int grp, __bf16* k_lds, __bf16* v_lds, int32_t* page_lds) {
     constexpr int KPITCH = 2 * 32 * NCH + 8;          // elements per key row in LDS (both maps)
     constexpr int VPITCH = TKEYS + 4;                 // elements per value channel row in LDS
-    __shared__ __attribute__((aligned(16))) __bf16 k_lds[TKEYS * KPITCH];
-    __shared__ __attribute__((aligned(16))) __bf16 v_lds[16 * NDB * VPITCH];
     const int D = a.head_dim, V = a.value_dim, P = a.page_size;
     const int g = a.q_heads / a.kv_heads;
     const int head_sets = (g + heads_per_wg - 1) / heads_per_wg;
-    const int grp = blockIdx.x, kvh = blockIdx.y / head_sets, head_set = blockIdx.y % head_sets;
+    const int kvh = blockIdx.y / head_sets, head_set = blockIdx.y % head_sets;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, b = lane >> 4;
     const int row0 = group_row0[grp], ntok = group_ntok[grp];
@@ -304,40 +303,92 @@ __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffArgs a, c
     const int split = blockIdx.z;
     const int k_lo = a.max_splits > 1 ? split * a.split_keys : 0;
     const int k_hi = a.max_splits > 1 ? min(ke, (split + 1) * a.split_keys) : ke;
-    for (int tb = k_lo; tb < k_hi; tb += TKEYS) {
-        __syncthreads();                              // the tile before has been read
-        for (int ci = threadIdx.x; ci < k_chunks; ci += 256) {
-            const int key = ci / (2 * D / 8), c8 = ci % (2 * D / 8);
-            const int kp = tb + key;
-            bf16x8 kv = zero8;
-            if (kp < k_hi) {
-                const int block = kp / P;
-                const int page = block < a.max_blocks ? table[block] : -1;
-                if (page >= 0)
-                    kv = *reinterpret_cast<const bf16x8*>(kp_base + (((size_t)page * a.kv_heads + kvh) * P + kp % P) * (2 * D) + 8 * c8);
-            }
-            // (map m's channel d goes to column m * 32 NCH + d, so that both maps start a row of chunks)
-            const int ch = 8 * c8, map = ch >= D ? 1 : 0;
-            *reinterpret_cast<bf16x8*>(&k_lds[key * KPITCH + map * 32 * NCH + (ch - map * D)]) = kv;
+    if (k_lo >= k_hi) return;                         // (a range beyond the group's keys: the merge does not read it)
+    // page ids of the range first, so that a tile's loads do not wait for a load of the block table
+    const int first_page = k_lo / P;                  // (k_lo is a multiple of 64; pages of 8 k tokens)
+    {
+        const int n_pages = min(TILES_PAGE_CACHE, (k_hi + P - 1) / P - first_page);
+        for (int i = threadIdx.x; i < n_pages; i += 256) page_lds[i] = first_page + i < a.max_blocks ? table[first_page + i] : -1;
+        __syncthreads();
+    }
+    // (no load from the block table here: a global load behind a branch makes the compiler wait for every load in
+    // flight, one tile's loads would then go out one after the other; the host keeps a range within the cache)
+    const bool pow2 = (P & (P - 1)) == 0;
+    const int pshift = __ffs(P) - 1;
+    auto block_of = [&](int kp) { return pow2 ? kp >> pshift : kp / P; };
+    auto within = [&](int kp) { return pow2 ? kp & (P - 1) : kp % P; };
+    auto page_of = [&](int kp) {
+        const int page = page_lds[min(max(block_of(kp) - first_page, 0), TILES_PAGE_CACHE - 1)];
+        return kp < k_hi ? page : -1;
+    };
+    // what a thread stages does not change from tile to tile
+    constexpr int KST = NCH, VST = (NDB + 3) / 4;     // 16-byte chunks a thread stages per tile
+    int k_key[KST], k_goff[KST], k_loff[KST], v_ch[VST], v_key[VST], v_loff[VST];
+    bool k_mine[KST], v_mine[VST];
+#pragma unroll
+    for (int i = 0; i < KST; ++i) {
+        k_mine[i] = (int)threadIdx.x + 256 * i < k_chunks;
+        const int ci = min((int)threadIdx.x + 256 * i, k_chunks - 1);
+        const int key = ci / (2 * D / 8), ch = 8 * (ci % (2 * D / 8)), map = ch >= D ? 1 : 0;
+        k_key[i] = key;
+        k_goff[i] = ch;
+        // (map m's channel d goes to column m * 32 NCH + d, so that both maps start a row of chunks)
+        k_loff[i] = key * KPITCH + map * 32 * NCH + (ch - map * D);
+    }
+#pragma unroll
+    for (int i = 0; i < VST; ++i) {
+        v_mine[i] = (int)threadIdx.x + 256 * i < v_chunks;
+        const int ci = min((int)threadIdx.x + 256 * i, v_chunks - 1);
+        v_ch[i] = ci >> 2;
+        v_key[i] = 8 * (ci & 3);
+        v_loff[i] = (ci >> 2) * VPITCH + 8 * (ci & 3);
+    }
+    struct Staged {                                   // one tile on its way: registers between memory and LDS
+        bf16x8 k[KST], v[VST];
+        int tb, ok;                                   // bit i: chunk i of the keys, bit 16 + i: of the values, is there
+    };
+    // global -> registers, no branch around a load (a load behind a branch makes the compiler wait for every load in
+    // flight): addresses are clamped to memory that exists, what must read as zero is zeroed on the way to LDS
+    auto fetch = [&](int tb, Staged& st) {
+        st.tb = tb;
+        st.ok = 0;
+#pragma unroll
+        for (int i = 0; i < KST; ++i) {
+            const int kp = tb + k_key[i];
+            const int page = page_of(kp);
+            if (page >= 0 && k_mine[i]) st.ok |= 1 << i;
+            st.k[i] = *reinterpret_cast<const bf16x8*>(kp_base + (((size_t)max(page, 0) * a.kv_heads + kvh) * P + within(kp)) * (2 * D) + k_goff[i]);
         }
-        for (int ci = threadIdx.x; ci < v_chunks; ci += 256) {
-            const int d = ci >> 2, q4 = ci & 3;
-            const int kp = tb + 8 * q4;
-            bf16x8 v = zero8;
-            if (kp < k_hi) {
-                const int block = kp / P;
-                const int page = block < a.max_blocks ? table[block] : -1;
-                if (page >= 0)
-                    v = *reinterpret_cast<const bf16x8*>(vp_base + (((size_t)page * a.kv_heads + kvh) * V + d) * P + kp % P);
+#pragma unroll
+        for (int i = 0; i < VST; ++i) {
+            const int kp = tb + v_key[i];
+            const int page = page_of(kp);
+            if (page >= 0 && v_mine[i]) st.ok |= 1 << (16 + i);
+            st.v[i] = *reinterpret_cast<const bf16x8*>(vp_base + (((size_t)max(page, 0) * a.kv_heads + kvh) * V + v_ch[i]) * P + within(kp));
+        }
+    };
+    auto stash = [&](const Staged& st) {              // registers -> LDS
+#pragma unroll
+        for (int i = 0; i < KST; ++i) {
+            if (!k_mine[i]) continue;
+            *reinterpret_cast<bf16x8*>(&k_lds[k_loff[i]]) = ((st.ok >> i) & 1) ? st.k[i] : zero8;
+        }
+#pragma unroll
+        for (int i = 0; i < VST; ++i) {
+            if (!v_mine[i]) continue;
+            bf16x8 v = ((st.ok >> (16 + i)) & 1) ? st.v[i] : zero8;
+            const int key0 = st.tb + v_key[i];
+            if (key0 + 8 > k_hi) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e)           // keys that are not written yet count as zero
-                    if (kp + e >= k_hi) v[e] = (__bf16)0.f;
+                    if (key0 + e >= k_hi) v[e] = (__bf16)0.f;
             }
-            *reinterpret_cast<bf16x4*>(&v_lds[d * VPITCH + 8 * q4]) = bf16x4{v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<bf16x4*>(&v_lds[d * VPITCH + 8 * q4 + 4]) = bf16x4{v[4], v[5], v[6], v[7]};
+            *reinterpret_cast<bf16x4*>(&v_lds[v_loff[i]]) = bf16x4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<bf16x4*>(&v_lds[v_loff[i] + 4]) = bf16x4{v[4], v[5], v[6], v[7]};
         }
-        __syncthreads();
-        if (!wave_active || tb >= wave_hi) continue;
+    };
+    auto compute = [&](int tb) {
+        if (!wave_active || tb >= wave_hi) return;
         const bool interior = tb + TKEYS <= wave_first_kend;
 #pragma unroll
         for (int map = 0; map < 2; ++map) {
@@ -370,6 +421,7 @@ __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffArgs a, c
                                    fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
             tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLR_WAVE));
             tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLR_WAVE));
+            // (the running maximum rarely moves after the first tiles: rescale only when it does, for any column)
             if (__builtin_amdgcn_ballot_w64(tile_max > m_run[map]) != 0) {
                 const float m_new = fmaxf(m_run[map], tile_max);
                 const float corr = m_new > -INFINITY ? __builtin_amdgcn_exp2f(m_run[map] - m_new) : 1.f;
@@ -400,6 +452,25 @@ __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffArgs a, c
                 o[map][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[map][db], 0, 0, 0);
             }
         }
+    };
+    // Two tiles are on their way from memory while one is multiplied: with one, a workgroup's time a tile is the
+    // memory's answer time.  (Fetches are unconditional, clamped to the last tile.)
+    const int tb_last = k_lo + ((k_hi - k_lo - 1) / TKEYS) * TKEYS;
+    Staged sa, sb;
+    fetch(k_lo, sa);
+    fetch(min(k_lo + TKEYS, tb_last), sb);
+    for (int tb = k_lo; tb < k_hi; tb += 2 * TKEYS) {
+        __syncthreads();                              // the tile before has been read
+        stash(sa);
+        __syncthreads();
+        fetch(min(tb + 2 * TKEYS, tb_last), sa);
+        compute(tb);
+        if (tb + TKEYS >= k_hi) break;
+        __syncthreads();
+        stash(sb);
+        __syncthreads();
+        fetch(min(tb + 3 * TKEYS, tb_last), sb);
+        compute(tb + TKEYS);
     }
 #pragma unroll
     for (int map = 0; map < 2; ++map) {
@@ -459,15 +530,27 @@ __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffArgs a, c
     }
 }
 
+template <int NCH, int NDB>
+__global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffArgs a, const int32_t* __restrict__ group_row0,
+                                                                   const int32_t* __restrict__ group_ntok, int groups,
+                                                                   int heads_per_wg, int token_blocks) {
+    __shared__ __attribute__((aligned(16))) __bf16 k_lds[TKEYS * (2 * 32 * NCH + 8)];
+    __shared__ __attribute__((aligned(16))) __bf16 v_lds[16 * NDB * (TKEYS + 4)];
+    __shared__ int32_t page_lds[TILES_PAGE_CACHE];
+    // (the longest groups of a prompt first: the workgroups that start last are the short ones)
+    diff_tiles_group<NCH, NDB>(a, group_row0, group_ntok, heads_per_wg, token_blocks, groups - 1 - (int)blockIdx.x, k_lds, v_lds,
+                               page_lds);
+}
+
 template <int NCH>
 static int launch_tiles(const DiffArgs& a, const int32_t* row0, const int32_t* ntok, int groups, int hpw, int tbw,
                         hipStream_t stream) {
     const int g = a.q_heads / a.kv_heads;
     dim3 grid(groups, a.kv_heads * ((g + hpw - 1) / hpw), a.max_splits);
     const int ndb = (a.value_dim + 15) / 16;
-    if (ndb <= 2) diff_attention_tiles_kernel<NCH, 2><<<grid, 256, 0, stream>>>(a, row0, ntok, hpw, tbw);
-    else if (ndb <= 4) diff_attention_tiles_kernel<NCH, 4><<<grid, 256, 0, stream>>>(a, row0, ntok, hpw, tbw);
-    else diff_attention_tiles_kernel<NCH, 8><<<grid, 256, 0, stream>>>(a, row0, ntok, hpw, tbw);
+    if (ndb <= 2) diff_attention_tiles_kernel<NCH, 2><<<grid, 256, 0, stream>>>(a, row0, ntok, groups, hpw, tbw);
+    else if (ndb <= 4) diff_attention_tiles_kernel<NCH, 4><<<grid, 256, 0, stream>>>(a, row0, ntok, groups, hpw, tbw);
+    else diff_attention_tiles_kernel<NCH, 8><<<grid, 256, 0, stream>>>(a, row0, ntok, groups, hpw, tbw);
     return (int)hipGetLastError();
 }
 #endif
@@ -512,16 +595,20 @@ int mlr_diff_attention(const void* q, long q_stride, const void* k_pages, const 
 // 16 * (4 / min(4, q_heads / kv_heads)) tokens, single tokens and short portions in smaller ones.  `group_tokens`:
 // the most tokens of a group.  With max_splits > 1 every group's keys are cut into ranges of split_keys (a
 // multiple of 64) whose partial results [groups * group_tokens, q_heads * 2, max_splits, value_dim + 2] are merged
-// by the kernel that also serves the scalar path.  Returns -10 where the sizes are not taken.
+// by the kernel that also serves the scalar path.  `max_context`: no token of the step lies at or beyond it.
+// Returns -10 where the sizes are not taken.
 int mlr_diff_attention_tiles(const void* q, long q_stride, const void* k_pages, const void* v_pages,
                              const int32_t* block_table, int max_blocks, const int32_t* slots, const int32_t* positions,
                              const void* gate, long gate_stride, void* out, float* partial, const int32_t* group_row0,
                              const int32_t* group_ntok, int groups, int group_tokens, int q_heads, int kv_heads,
                              int head_dim, int value_dim, int page_size, float scale, float softcap, float temp_coef,
                              float temp_every, float lam, float out_scale, float eps, int split_keys, int max_splits,
-                             hipStream_t stream) {
+                             int max_context, hipStream_t stream) {
 #if MLR_BF16
     if (groups <= 0) return 0;
+    // the keys one workgroup walks (a range, or without ranges the longest context of the step) lie in at most
+    // TILES_PAGE_CACHE pages, whose ids it keeps in LDS
+    if (((max_splits > 1 ? split_keys : max_context) + page_size - 1) / page_size + 1 > TILES_PAGE_CACHE) return -4;
     if (head_dim % 16 != 0 || head_dim > 128 || value_dim % 16 != 0 || value_dim > 128 || page_size % 8 != 0 ||
         q_heads % kv_heads != 0 || q_stride % 8 != 0 || (gate != nullptr && gate_stride % 4 != 0)) return -10;
     if (max_splits < 1) max_splits = 1;

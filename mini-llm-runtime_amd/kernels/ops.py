@@ -900,6 +900,13 @@ class Kernels:
                 and value_dim <= 128 and page_size % 8 == 0 and q_heads % kv_heads == 0 and q_stride % 8 == 0
                 and gate_stride % 4 == 0)
 
+    DIFF_TILES_PAGES = 2048
+
+    @classmethod
+    def diff_tiles_reach(cls, page_size):
+        """The most keys that one workgroup of the matrix-core kernel walks (it keeps their pages' ids in LDS)."""
+        return (cls.DIFF_TILES_PAGES - 2) * page_size
+
     @staticmethod
     def diff_tiles_group_tokens(q_heads, kv_heads):
         """Tokens of a prompt portion that one workgroup of the matrix-core kernel takes: its four wavefronts serve
@@ -909,9 +916,12 @@ class Kernels:
     @timed("attention")
     def diff_attention_tiles(self, q, k_pages, v_pages, block_table, slots, positions, gate, out, partial, group_row0,
                              group_ntok, groups, group_tokens, q_heads, kv_heads, head_dim, value_dim, page_size, scale, lam,
-                             out_scale, eps, softcap=None, temp_coef=0.0, temp_every=1.0, split_keys=0, max_splits=1):
+                             out_scale, eps, softcap=None, temp_coef=0.0, temp_every=1.0, split_keys=0, max_splits=1,
+                             max_context=None):
         """As `diff_attention` for the rows of `groups` groups of consecutive tokens of one request each (first row,
-        number of tokens: device int32 vectors; at most `group_tokens` tokens a group), on the matrix cores."""
+        number of tokens: device int32 vectors; at most `group_tokens` tokens a group), on the matrix cores.
+        `max_context`: a bound on the step's positions + 1 (default: what the block table can hold); the keys that one
+        workgroup walks -- a key range, or all of them -- must lie in `DIFF_TILES_PAGES` pages at most."""
         rows = q.shape[0]
         qs = self._columns(q, "q", self.dtype, rows, q_heads * 2 * head_dim)
         gs = self._columns(gate, "gate", self.dtype, rows, q_heads * value_dim) if gate is not None else 0
@@ -934,13 +944,17 @@ class Kernels:
             _need(split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0 and max_splits <= MAX_KEY_SPLITS,
                   "diff_attention_tiles: key ranges must be multiples of 64 keys, at most 1024 of them")
         _need(kv_heads * 4 <= 65535 and max_splits <= 65535, "diff_attention_tiles: grid too large")
+        if max_context is None:
+            max_context = block_table.shape[1] * page_size
+        _need(self.diff_tiles_reach(page_size) >= (split_keys if max_splits > 1 else max_context),
+              "diff_attention_tiles: one workgroup would walk more pages than it keeps ids of; cut the keys into ranges")
         fn = self._lib("diff_attention").mlr_diff_attention_tiles
         _ok(fn(_p(q), ctypes.c_long(qs), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
                _p(positions), _p(gate), ctypes.c_long(gs), _p(out), _p(partial if max_splits > 1 else None), _p(group_row0),
                _p(group_ntok), _c_int(groups), _c_int(group_tokens), _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim),
                _c_int(value_dim), _c_int(page_size), _c_float(scale), _c_float(softcap or 0.0), _c_float(temp_coef),
                _c_float(temp_every), _c_float(lam), _c_float(out_scale), _c_float(eps), _c_int(split_keys),
-               _c_int(max_splits), _stream()), "diff_attention_tiles")
+               _c_int(max_splits), _c_int(max_context), _stream()), "diff_attention_tiles")
 
     # -- sampling ----------------------------------------------------------------------------
     def sample_scratch(self, rows):

@@ -43,6 +43,7 @@ class DiffAttention:
         self.proj = self.o = None
         self.lam = None
         self._partial_floats = PARTIAL_CAP
+        self._page_size = 16
 
     def weight_specs(self):
         s = self.spec
@@ -107,13 +108,18 @@ class DiffAttention:
         the partial results fit `budget` floats."""
         s = self.spec
         base, longest = ctx.split_keys, ctx.max_context
-        if base <= 0 or longest <= base or units >= ctx.target_workgroups:
+        reach = ctx.kernels.diff_tiles_reach(self._page_size)       # the most keys one workgroup walks
+        forced = longest > reach
+        if base <= 0 and forced:
+            raise PartError(f"a context of {longest} tokens needs key ranges (split_keys > 0): one workgroup walks {reach} keys")
+        if base <= 0 or longest <= base or (units >= ctx.target_workgroups and not forced):
             return 0, 1
         keys = base
-        while keys * 2 < longest and units * (-(-longest // (keys * 2))) >= ctx.target_workgroups:
+        while keys * 2 < longest and keys * 2 <= reach and (units * (-(-longest // (keys * 2))) >= ctx.target_workgroups or
+                                                             (forced and units >= ctx.target_workgroups)):
             keys *= 2
         numel = lambda k: ctx.kernels.diff_partial_numel(places, s.q_heads, s.value_dim, -(-longest // k))
-        while (numel(keys) > budget or -(-longest // keys) > 1024) and keys < longest:
+        while (numel(keys) > budget or -(-longest // keys) > 1024) and keys < longest and keys * 2 <= reach:
             keys *= 2
         splits = -(-longest // keys)
         return (keys, splits) if splits > 1 else (0, 1)
@@ -124,6 +130,7 @@ class DiffAttention:
         s = self.spec
         k = ctx.kernels
         tokens = k.diff_tiles_group_tokens(s.q_heads, s.kv_heads)
+        self._page_size = view.page_size
         small, big, _ = ctx.token_groups(SMALL_GROUP, tokens // SMALL_GROUP)
         temp = s.q_temperature
         g = s.q_heads // s.kv_heads
@@ -137,7 +144,8 @@ class DiffAttention:
                                    attn, partial, first, count, n, group_tokens, s.q_heads, s.kv_heads, s.head_dim,
                                    s.value_dim, view.page_size, float(s.scale), self.lam, float(s.out_scale), float(s.eps),
                                    softcap=s.softcap, temp_coef=temp.coef if temp else 0.0,
-                                   temp_every=temp.every if temp else 1.0, split_keys=split_keys, max_splits=splits)
+                                   temp_every=temp.every if temp else 1.0, split_keys=split_keys, max_splits=splits,
+                                   max_context=ctx.max_context)
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
