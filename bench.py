@@ -19,6 +19,9 @@ many gigabytes).  Every runner is built with the product's own defaults.  One JS
     share of its roofline; the 64 requests of a block are filled once and serve all of its measurements.
     `--size 32b --only mixed` measures the mixed step alone.
   * --profile: time per kernel class (event pairs around every launch, steps run eagerly) beside the line.
+  * --only taletar: a line of its own: prefill and decode of Taletar models (Mamba-2, differential attention and
+    gated linear attention layers) at two layer sizes beside a Qwen3 dense model of the same width, heads,
+    feed-forward and layers, with milliseconds per kernel class.  The default workload is not touched by it.
 """
 import argparse
 import json
