@@ -244,29 +244,39 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 // head_dim and value_dim multiples of 16, the page size a multiple of 8.
 template <int NCH, int NDB>
 __device__ __forceinline__ void diff_tiles_group(const DiffArgs& a, const int32_t* __restrict__ group_row0,
-                                                 const int32_t* __restrict__ group_ntok, int heads_per_wg, int token_blocks,
-                                                 int grp, __bf16* k_lds, __bf16* v_lds, int32_t* page_lds) {
+                                                 const int32_t* __restrict__ group_ntok, int col_heads, int wave_heads,
+                                                 int token_blocks, int map_split, int grp, __bf16* k_lds, __bf16* v_lds,
+                                                 int32_t* page_lds) {
     constexpr int KPITCH = 2 * 32 * NCH + 8;          // elements per key row in LDS (both maps)
     constexpr int VPITCH = TKEYS + 4;                 // elements per value channel row in LDS
     const int D = a.head_dim, V = a.value_dim, P = a.page_size;
     const int g = a.q_heads / a.kv_heads;
+    // The 16 columns of a wavefront: `col_heads` query heads of the kv head side by side for each of 16 / col_heads
+    // tokens (prompt portions: one head, 16 tokens; single tokens and short portions: up to four heads of each
+    // token, so that one wavefront serves what four would).  The four wavefronts: `wave_heads` sets of heads x
+    // `token_blocks` blocks of tokens; with `map_split` (partial results only) two sets of heads and blocks, wavefronts
+    // 0 and 1 taking map 1 and wavefronts 2 and 3 map 2 of the same columns: half the chain of instructions a tile.
+    const int heads_per_wg = col_heads * wave_heads;
     const int head_sets = (g + heads_per_wg - 1) / heads_per_wg;
     const int kvh = blockIdx.y / head_sets, head_set = blockIdx.y % head_sets;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = map_split ? (int)((threadIdx.x >> 6) & 1) : (int)(threadIdx.x >> 6);
+    const int my_map = threadIdx.x >> 7;              // (map_split only)
     const int col = lane & 15, b = lane >> 4;
     const int row0 = group_row0[grp], ntok = group_ntok[grp];
     const int slot = a.slots[row0], pos0 = a.positions[row0];
-    const int hh = head_set * heads_per_wg + wave % heads_per_wg;         // head within the kv head's set
-    const int tblock = wave / heads_per_wg;
+    const int tokens_per_wave = 16 / col_heads;
+    const int head0 = (head_set * wave_heads + wave % wave_heads) * col_heads;      // the wavefront's first head in the set
+    const int hh = head0 + col % col_heads;
+    const int tblock = wave / wave_heads;
     const int head = kvh * g + hh;
-    const int tok = tblock * 16 + col;
-    const bool wave_active = tblock < token_blocks && hh < g && tblock * 16 < ntok;
-    const bool col_valid = wave_active && tok < ntok;
+    const int tok = tblock * tokens_per_wave + col / col_heads;
+    const bool wave_active = tblock < token_blocks && head0 < g && tblock * tokens_per_wave < ntok;
+    const bool col_valid = wave_active && col < tokens_per_wave * col_heads && hh < g && tok < ntok;
     const int pos = pos0 + tok;
     const int kend_c = col_valid ? pos + 1 : 0;       // keys this column sees: [0, kend_c)
     const int ke = pos0 + ntok;                       // keys the workgroup walks: [0, ke)
-    const int wave_hi = wave_active ? pos0 + min(ntok, tblock * 16 + 16) : 0;
-    const int wave_first_kend = pos0 + tblock * 16 + 1;
+    const int wave_hi = wave_active ? pos0 + min(ntok, tblock * tokens_per_wave + tokens_per_wave) : 0;
+    const int wave_first_kend = pos0 + tblock * tokens_per_wave + 1;
     const __bf16* q = reinterpret_cast<const __bf16*>(a.q);
     const __bf16* kp_base = reinterpret_cast<const __bf16*>(a.k_pages);
     const __bf16* vp_base = reinterpret_cast<const __bf16*>(a.v_pages);
@@ -392,6 +402,7 @@ __device__ __forceinline__ void diff_tiles_group(const DiffArgs& a, const int32_
         const bool interior = tb + TKEYS <= wave_first_kend;
 #pragma unroll
         for (int map = 0; map < 2; ++map) {
+            if (map_split && map != my_map) continue;
             floatx4 s[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -477,12 +488,13 @@ __device__ __forceinline__ void diff_tiles_group(const DiffArgs& a, const int32_
         l_run[map] += __shfl_xor(l_run[map], 16, MLR_WAVE);
         l_run[map] += __shfl_xor(l_run[map], 32, MLR_WAVE);
     }
-    if (a.max_splits > 1) {
+    if (a.partial != nullptr) {
         // (max, sum, weighted values) of this key range, the maximum back in the natural domain
         if (!col_valid) return;
         const size_t place = (size_t)grp * a.group_tokens + tok;
 #pragma unroll
         for (int map = 0; map < 2; ++map) {
+            if (map_split && map != my_map) continue;
             float* dst = a.partial + ((place * a.q_heads * 2 + head * 2 + map) * a.max_splits + split) * (V + 2);
 #pragma unroll
             for (int db = 0; db < NDB; ++db) {
@@ -533,24 +545,25 @@ __device__ __forceinline__ void diff_tiles_group(const DiffArgs& a, const int32_
 template <int NCH, int NDB>
 __global__ __launch_bounds__(256) void diff_attention_tiles_kernel(DiffArgs a, const int32_t* __restrict__ group_row0,
                                                                    const int32_t* __restrict__ group_ntok, int groups,
-                                                                   int heads_per_wg, int token_blocks) {
+                                                                   int col_heads, int wave_heads, int token_blocks,
+                                                                   int map_split) {
     __shared__ __attribute__((aligned(16))) __bf16 k_lds[TKEYS * (2 * 32 * NCH + 8)];
     __shared__ __attribute__((aligned(16))) __bf16 v_lds[16 * NDB * (TKEYS + 4)];
     __shared__ int32_t page_lds[TILES_PAGE_CACHE];
     // (the longest groups of a prompt first: the workgroups that start last are the short ones)
-    diff_tiles_group<NCH, NDB>(a, group_row0, group_ntok, heads_per_wg, token_blocks, groups - 1 - (int)blockIdx.x, k_lds, v_lds,
-                               page_lds);
+    diff_tiles_group<NCH, NDB>(a, group_row0, group_ntok, col_heads, wave_heads, token_blocks, map_split,
+                               groups - 1 - (int)blockIdx.x, k_lds, v_lds, page_lds);
 }
 
 template <int NCH>
-static int launch_tiles(const DiffArgs& a, const int32_t* row0, const int32_t* ntok, int groups, int hpw, int tbw,
-                        hipStream_t stream) {
+static int launch_tiles(const DiffArgs& a, const int32_t* row0, const int32_t* ntok, int groups, int ch, int wh, int tbw,
+                        int ms, hipStream_t stream) {
     const int g = a.q_heads / a.kv_heads;
-    dim3 grid(groups, a.kv_heads * ((g + hpw - 1) / hpw), a.max_splits);
+    dim3 grid(groups, a.kv_heads * ((g + ch * wh - 1) / (ch * wh)), a.max_splits);
     const int ndb = (a.value_dim + 15) / 16;
-    if (ndb <= 2) diff_attention_tiles_kernel<NCH, 2><<<grid, 256, 0, stream>>>(a, row0, ntok, groups, hpw, tbw);
-    else if (ndb <= 4) diff_attention_tiles_kernel<NCH, 4><<<grid, 256, 0, stream>>>(a, row0, ntok, groups, hpw, tbw);
-    else diff_attention_tiles_kernel<NCH, 8><<<grid, 256, 0, stream>>>(a, row0, ntok, groups, hpw, tbw);
+    if (ndb <= 2) diff_attention_tiles_kernel<NCH, 2><<<grid, 256, 0, stream>>>(a, row0, ntok, groups, ch, wh, tbw, ms);
+    else if (ndb <= 4) diff_attention_tiles_kernel<NCH, 4><<<grid, 256, 0, stream>>>(a, row0, ntok, groups, ch, wh, tbw, ms);
+    else diff_attention_tiles_kernel<NCH, 8><<<grid, 256, 0, stream>>>(a, row0, ntok, groups, ch, wh, tbw, ms);
     return (int)hipGetLastError();
 }
 #endif
@@ -614,19 +627,27 @@ int mlr_diff_attention_tiles(const void* q, long q_stride, const void* k_pages, 
     if (max_splits < 1) max_splits = 1;
     if (max_splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % TILE_KEYS != 0 ||
                            max_splits > COMBINE_MAX_SPLITS)) return -2;
+    // (partial given with one range: the kernel still leaves partial results and the merge kernel finishes the head)
     const int g = q_heads / kv_heads;
-    const int hpw = g < 4 ? g : 4, tbw = 4 / hpw;
-    if (group_tokens < 1 || group_tokens > 16 * tbw) return -3;
+    // groups of up to four tokens: up to four heads of a token side by side in a wavefront's columns; longer groups
+    // (prompt portions): a head a wavefront, 16 tokens in its columns
+    const int ch = group_tokens <= 4 ? (g < 4 ? g : 4) : 1;
+    const int sets = (g + ch - 1) / ch;
+    // (with partial results, small groups give each map wavefronts of its own: two layout places instead of four)
+    const int ms = (group_tokens <= 4 && partial != nullptr) ? 1 : 0;
+    const int places = ms ? 2 : 4;
+    const int wh = sets < places ? sets : places, tbw = places / wh;
+    if (group_tokens < 1 || group_tokens > (16 / ch) * tbw) return -3;
     DiffArgs a{(const elem_t*)q, q_stride, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots, positions,
                (const elem_t*)gate, gate_stride, (elem_t*)out, partial, max_blocks, q_heads, kv_heads, head_dim, value_dim,
                page_size, split_keys, max_splits, scale, softcap, temp_coef, temp_every, lam, out_scale, eps,
                group_row0, group_ntok, group_tokens};
     const int nch = (head_dim + 31) / 32;
     int err;
-    if (nch == 1) err = launch_tiles<1>(a, group_row0, group_ntok, groups, hpw, tbw, stream);
-    else if (nch == 2) err = launch_tiles<2>(a, group_row0, group_ntok, groups, hpw, tbw, stream);
-    else err = launch_tiles<4>(a, group_row0, group_ntok, groups, hpw, tbw, stream);
-    if (err != 0 || max_splits == 1) return err;
+    if (nch == 1) err = launch_tiles<1>(a, group_row0, group_ntok, groups, ch, wh, tbw, ms, stream);
+    else if (nch == 2) err = launch_tiles<2>(a, group_row0, group_ntok, groups, ch, wh, tbw, ms, stream);
+    else err = launch_tiles<4>(a, group_row0, group_ntok, groups, ch, wh, tbw, ms, stream);
+    if (err != 0 || partial == nullptr) return err;
     diff_attention_combine_kernel<<<dim3(groups * group_tokens, q_heads), 64, 0, stream>>>(a);
     return (int)hipGetLastError();
 #else

@@ -937,10 +937,14 @@ class Kernels:
         _tensor(group_ntok, "group_ntok", torch.int32, (groups,))
         _need(1 <= group_tokens <= self.diff_tiles_group_tokens(q_heads, kv_heads), "diff_attention_tiles: group too large")
         max_splits = max(1, max_splits)
-        if max_splits > 1:
+        # partial results: with key ranges always; without them for groups of up to four tokens when `partial` is
+        # given (the two maps then run in wavefronts of their own and the merge kernel finishes the head)
+        through_partial = max_splits > 1 or (partial is not None and group_tokens <= 4)
+        if through_partial:
             _tensor(partial, "partial", torch.float32, ndim=1)
             _need(partial.numel() >= self.diff_partial_numel(groups * group_tokens, q_heads, value_dim, max_splits),
                   "diff_attention_tiles: partial too small")
+        if max_splits > 1:
             _need(split_keys > 0 and split_keys % ATTENTION_TILE_KEYS == 0 and max_splits <= MAX_KEY_SPLITS,
                   "diff_attention_tiles: key ranges must be multiples of 64 keys, at most 1024 of them")
         _need(kv_heads * 4 <= 65535 and max_splits <= 65535, "diff_attention_tiles: grid too large")
@@ -950,7 +954,7 @@ class Kernels:
               "diff_attention_tiles: one workgroup would walk more pages than it keeps ids of; cut the keys into ranges")
         fn = self._lib("diff_attention").mlr_diff_attention_tiles
         _ok(fn(_p(q), ctypes.c_long(qs), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
-               _p(positions), _p(gate), ctypes.c_long(gs), _p(out), _p(partial if max_splits > 1 else None), _p(group_row0),
+               _p(positions), _p(gate), ctypes.c_long(gs), _p(out), _p(partial if through_partial else None), _p(group_row0),
                _p(group_ntok), _c_int(groups), _c_int(group_tokens), _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim),
                _c_int(value_dim), _c_int(page_size), _c_float(scale), _c_float(softcap or 0.0), _c_float(temp_coef),
                _c_float(temp_every), _c_float(lam), _c_float(out_scale), _c_float(eps), _c_int(split_keys),

@@ -140,8 +140,12 @@ class DiffAttention:
             if n == 0:
                 continue
             split_keys, splits = self._tile_splits(ctx, n * per_group, n * group_tokens, partial.numel())
+            # (single tokens and short portions always leave partial results, where their room allows: the two maps
+            # of a head then run side by side and the merge kernel finishes the head)
+            through = splits > 1 or (group_tokens == SMALL_GROUP and
+                                     k.diff_partial_numel(n * group_tokens, s.q_heads, s.value_dim, 1) <= partial.numel())
             k.diff_attention_tiles(q, view.tensors["k"], view.tensors["v"], view.block_table, ctx.slots, ctx.positions, gate,
-                                   attn, partial, first, count, n, group_tokens, s.q_heads, s.kv_heads, s.head_dim,
+                                   attn, partial if through else None, first, count, n, group_tokens, s.q_heads, s.kv_heads, s.head_dim,
                                    s.value_dim, view.page_size, float(s.scale), self.lam, float(s.out_scale), float(s.eps),
                                    softcap=s.softcap, temp_coef=temp.coef if temp else 0.0,
                                    temp_every=temp.every if temp else 1.0, split_keys=split_keys, max_splits=splits,
