@@ -416,6 +416,141 @@ __global__ __launch_bounds__(256) void gated_part_norm_kernel(const float* __res
     }
 }
 
+#if MLR_BF16
+// The same three kernels with 16 bytes per lane and access (bfloat16 engine, widths in multiples of 8).
+__global__ __launch_bounds__(256) void add2_rmsnorm2_vec_kernel(float* __restrict__ h, const elem_t* __restrict__ d1,
+                                                                const elem_t* __restrict__ d2, const float* __restrict__ w1,
+                                                                const float* __restrict__ w2, elem_t* __restrict__ out1,
+                                                                elem_t* __restrict__ out2, int width, float eps) {
+    __shared__ float scratch[16];
+    const size_t r = blockIdx.x;
+    float* hrow = h + r * width;
+    float sum = 0.f;
+    for (int c = threadIdx.x * 8; c < width; c += 256 * 8) {
+        float x[8], a[8];
+        const float4 lo = *reinterpret_cast<const float4*>(hrow + c), hi = *reinterpret_cast<const float4*>(hrow + c + 4);
+        x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w; x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
+        if (d1 || d2) {
+            if (d1) load_vec(d1 + r * width + c, a);
+            else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a[e] = 0.f;
+            }
+            if (d2) {
+                float b[8];
+                load_vec(d2 + r * width + c, b);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a[e] += b[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] += a[e];
+            *reinterpret_cast<float4*>(hrow + c) = make_float4(x[0], x[1], x[2], x[3]);
+            *reinterpret_cast<float4*>(hrow + c + 4) = make_float4(x[4], x[5], x[6], x[7]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum += x[e] * x[e];
+    }
+    sum = block_sum(sum, scratch);
+    const float scale = 1.0f / sqrtf(sum / (float)width + eps);
+    for (int c = threadIdx.x * 8; c < width; c += 256 * 8) {       // (this thread wrote these elements of h itself)
+        float x[8], y[8];
+        const float4 lo = *reinterpret_cast<const float4*>(hrow + c), hi = *reinterpret_cast<const float4*>(hrow + c + 4);
+        x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w; x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = (x[e] * scale) * w1[c + e];
+        store_vec(out1 + r * width + c, y);
+        if (out2) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) y[e] = (x[e] * scale) * w2[c + e];
+            store_vec(out2 + r * width + c, y);
+        }
+    }
+}
+
+__global__ void clamped_glu_vec_kernel(const elem_t* __restrict__ gate_up, elem_t* __restrict__ act, int rows, int inter,
+                                       float limit, float slope) {
+    const int per_row = inter / 8;
+    const size_t total = (size_t)rows * per_row;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t m = i / per_row, f = (i % per_row) * 8;
+        float g[8], u[8], y[8];
+        load_vec(gate_up + m * 2 * inter + f, g);
+        load_vec(gate_up + m * 2 * inter + inter + f, u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float gg = fminf(g[e], limit), uu = fminf(fmaxf(u[e], -limit), limit);
+            y[e] = (gg / (1.0f + expf(-slope * gg))) * (uu + 1.0f);
+        }
+        store_vec(act + m * inter + f, y);
+    }
+}
+
+// WAVES wavefronts per (row, part): one for short parts, four (a workgroup) for long ones.
+template <int WAVES>
+__global__ __launch_bounds__(256) void gated_part_norm_vec_kernel(const float* __restrict__ y, const elem_t* __restrict__ gate,
+                                                                  long gate_stride, const float* __restrict__ weight,
+                                                                  elem_t* __restrict__ out, int rows, int width, int part,
+                                                                  int period, float eps, int gate_first, int gate_kind) {
+    __shared__ float scratch[16];
+    const int lane = WAVES == 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
+    const size_t unit = WAVES == 1 ? (size_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (size_t)blockIdx.x;
+    const int parts = width / part;
+    const bool live = unit < (size_t)rows * parts;
+    const size_t m = live ? unit / parts : 0;
+    const int c0 = live ? (int)(unit % parts) * part : 0;
+    const float* yrow = y + m * width;
+    const elem_t* grow = gate + m * gate_stride;
+    auto gated = [&](int c, float* v, bool before) {        // v = y[c .. c + 8), times the gate's activation when `before`
+        const float4 lo = *reinterpret_cast<const float4*>(yrow + c), hi = *reinterpret_cast<const float4*>(yrow + c + 4);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+        float z[8];
+        load_vec(grow + c, z);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float sg = 1.0f / (1.0f + expf(-z[e]));
+            z[e] = gate_kind == 0 ? z[e] * sg : sg;
+            if (before) v[e] *= z[e];
+        }
+        if (!before) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = z[e];         // (the caller wants the gate itself)
+        }
+    };
+    float sum = 0.f;
+    if (live)
+        for (int i = lane * 8; i < part; i += 64 * WAVES * 8) {
+            float v[8];
+            if (gate_first) gated(c0 + i, v, true);
+            else {
+                const float4 lo = *reinterpret_cast<const float4*>(yrow + c0 + i), hi = *reinterpret_cast<const float4*>(yrow + c0 + i + 4);
+                v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sum += v[e] * v[e];
+        }
+    sum = WAVES == 1 ? wave_sum(sum) : block_sum(sum, scratch);
+    if (!live) return;
+    const float scale = 1.0f / sqrtf(sum / (float)part + eps);
+    for (int i = lane * 8; i < part; i += 64 * WAVES * 8) {
+        const int c = c0 + i;
+        float v[8], o[8];
+        if (gate_first) {
+            gated(c, v, true);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (v[e] * scale) * weight[(c + e) % period];
+        } else {
+            float gt[8];
+            gated(c, gt, false);
+            const float4 lo = *reinterpret_cast<const float4*>(yrow + c), hi = *reinterpret_cast<const float4*>(yrow + c + 4);
+            v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = ((v[e] * scale) * weight[(c + e) % period]) * gt[e];
+        }
+        store_vec(out + m * width + c, o);
+    }
+}
+#endif
+
 static int grid_for(size_t count, int block) {
     size_t g = (count + block - 1) / block;
     return (int)(g > 65535 ? 65535 : (g == 0 ? 1 : g));
@@ -491,6 +626,13 @@ int mlr_add2_rmsnorm2(float* h, const void* d1, const void* d2, const float* w1,
                       int rows, int width, float eps, hipStream_t stream) {
     if (rows <= 0) return 0;
     if ((out2 == nullptr) != (w2 == nullptr)) return -1;
+#if MLR_BF16
+    if (width % 8 == 0) {
+        add2_rmsnorm2_vec_kernel<<<rows, 256, 0, stream>>>(h, (const elem_t*)d1, (const elem_t*)d2, w1, w2, (elem_t*)out1,
+                                                           (elem_t*)out2, width, eps);
+        return (int)hipGetLastError();
+    }
+#endif
     add2_rmsnorm2_kernel<<<rows, 256, 0, stream>>>(h, (const elem_t*)d1, (const elem_t*)d2, w1, w2, (elem_t*)out1,
                                                    (elem_t*)out2, width, eps);
     return (int)hipGetLastError();
@@ -504,6 +646,13 @@ int mlr_residual_add2(float* h, const void* d1, const void* d2, size_t count, hi
 
 int mlr_clamped_glu(const void* gate_up, void* act, int rows, int inter, float limit, float slope, hipStream_t stream) {
     if (rows <= 0) return 0;
+#if MLR_BF16
+    if (inter % 8 == 0) {
+        clamped_glu_vec_kernel<<<grid_for((size_t)rows * (inter / 8), 256), 256, 0, stream>>>((const elem_t*)gate_up, (elem_t*)act,
+                                                                                            rows, inter, limit, slope);
+        return (int)hipGetLastError();
+    }
+#endif
     clamped_glu_kernel<<<grid_for((size_t)rows * inter, 256), 256, 0, stream>>>((const elem_t*)gate_up, (elem_t*)act, rows,
                                                                               inter, limit, slope);
     return (int)hipGetLastError();
@@ -514,6 +663,21 @@ int mlr_gated_part_norm(const float* y, const void* gate, long gate_stride, cons
     if (rows <= 0) return 0;
     if (part <= 0 || width % part != 0 || period <= 0) return -1;
     const size_t units = (size_t)rows * (width / part);
+#if MLR_BF16
+    // (16-byte accesses: parts, the gate's rows and its first column at multiples of 8 elements)
+    if (part % 8 == 0 && gate_stride % 8 == 0 && ((uintptr_t)gate) % 16 == 0 && units < (1u << 31)) {
+        if (part >= 2048)
+            gated_part_norm_vec_kernel<4><<<(unsigned)units, 256, 0, stream>>>(y, (const elem_t*)gate, gate_stride, weight,
+                                                                              (elem_t*)out, rows, width, part, period, eps,
+                                                                              gate_first, gate_kind);
+        else
+            gated_part_norm_vec_kernel<1><<<(unsigned)((units + 3) / 4), 256, 0, stream>>>(y, (const elem_t*)gate, gate_stride,
+                                                                                          weight, (elem_t*)out, rows, width,
+                                                                                          part, period, eps, gate_first,
+                                                                                          gate_kind);
+        return (int)hipGetLastError();
+    }
+#endif
     gated_part_norm_kernel<<<(unsigned)((units + 3) / 4), 256, 0, stream>>>(y, (const elem_t*)gate, gate_stride, weight,
                                                                            (elem_t*)out, rows, width, part, period, eps,
                                                                            gate_first, gate_kind);

@@ -375,17 +375,18 @@ def test_differential_attention_against_the_plain_maps(dtype_name, path):
 
 
 @pytest.mark.parametrize("dtype_name", DTYPES)
-def test_row_kernels(dtype_name):
+@pytest.mark.parametrize("width,inter", [(90, 37), (96, 40), (2304, 8)])      # (scalar accesses; 16-byte ones; several turns a thread)
+def test_row_kernels(dtype_name, width, inter):
     from mini_llm_runtime_amd.kernels import Kernels
     dtype = DTYPES[dtype_name]
     k = Kernels(dtype)
     rng = np.random.default_rng(2)
     tol = 1e-5 if dtype_name == "float32" else 1e-2
-    m, width = 5, 90
+    m = 5
     h0 = rng.normal(size=(m, width))
     d1, d2 = rounded(rng.normal(size=(m, width)), dtype), rounded(rng.normal(size=(m, width)), dtype)
     w1, w2 = rng.normal(size=width), rng.normal(size=width)
-    for a, b, second in ((d1, d2, True), (d1, None, True), (None, None, False)):
+    for a, b, second in ((d1, d2, True), (d1, None, True), (None, d2, False), (None, None, False)):
         h = torch.from_numpy(h0).float().cuda()
         o1, o2 = torch.empty(m, width, dtype=dtype, device="cuda"), torch.empty(m, width, dtype=dtype, device="cuda")
         k.add2_rmsnorm2(h, a, b, torch.from_numpy(w1).float().cuda(), torch.from_numpy(w2).float().cuda() if second else None,
@@ -398,31 +399,44 @@ def test_row_kernels(dtype_name):
     h = torch.from_numpy(h0).float().cuda()
     k.residual_add2(h, d1, d2)
     np.testing.assert_allclose(h.double().cpu().numpy(), h0.astype(np.float32) + d1.double().cpu().numpy() + d2.double().cpu().numpy(), atol=1e-6)
-    gate_up = rounded(rng.normal(size=(m, 2 * 37)) * 2, dtype)
-    act = torch.empty(m, 37, dtype=dtype, device="cuda")
+    gate_up = rounded(rng.normal(size=(m, 2 * inter)) * 2, dtype)
+    act = torch.empty(m, inter, dtype=dtype, device="cuda")
     k.clamped_glu(gate_up, act, 0.8, 1.702)
     gu = gate_up.double().cpu().numpy()
-    eye = np.eye(37)
-    want = P.clamped_glu(np.concatenate([gu[:, :37], gu[:, 37:]], axis=1),
-                         {"gate": np.concatenate([eye, 0 * eye], axis=1), "up": np.concatenate([0 * eye, eye], axis=1), "down": eye},
+    eye = np.eye(inter)
+    want = P.clamped_glu(gu, {"gate": np.concatenate([eye, 0 * eye], axis=1), "up": np.concatenate([0 * eye, eye], axis=1), "down": eye},
                          dict(limit=0.8))
     np.testing.assert_allclose(act.double().cpu().numpy(), want, atol=tol, rtol=tol)
-    # the gated norm in parts: gate before the norm with a weight as wide as the row; after it with one as wide as a part
-    y = rng.normal(size=(m, 120))
-    wide = rounded(rng.normal(size=(m, 300)), dtype)
-    gate = wide[:, 100:220]
-    g64 = gate.double().cpu().numpy()
-    for part, period, first in ((40, 120, True), (120, 120, True), (30, 30, False), (1, 120, True)):
-        weight = rng.normal(size=period)
-        out = torch.empty(m, 120, dtype=dtype, device="cuda")
-        k.gated_part_norm(torch.from_numpy(y).float().cuda(), gate, torch.from_numpy(weight).float().cuda(), out, part, 1e-5,
-                          gate_first=first, gate_kind="silu")
-        x = y.astype(np.float32).astype(np.float64)
-        if first:
-            want = P.grouped_rms_norm(x * P.silu(g64), np.tile(weight, 120 // period), 120 // part, 1e-5)
-        else:
-            want = P.grouped_rms_norm(x, np.tile(weight, 120 // period), 120 // part, 1e-5) * P.silu(g64)
-        np.testing.assert_allclose(out.double().cpu().numpy(), want, atol=tol * np.abs(want).max(), rtol=tol)
+
+
+@pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("offset,total", [(100, 300), (96, 304)])              # the gate's columns: unaligned, aligned to 16 bytes
+def test_gated_norm_in_parts(dtype_name, offset, total):
+    """Gate before the norm with a weight as wide as the row; after it with one as wide as a part; parts of one value,
+    of a row, and long enough for a whole workgroup."""
+    from mini_llm_runtime_amd.kernels import Kernels
+    dtype = DTYPES[dtype_name]
+    k = Kernels(dtype)
+    rng = np.random.default_rng(6)
+    tol = 1e-5 if dtype_name == "float32" else 1e-2
+    m = 5
+    for width, cases in ((120, ((40, 120, True), (120, 120, True), (24, 24, False), (1, 120, True), (8, 8, False))),
+                         (4096, ((4096, 4096, True), (2048, 4096, True), (2048, 2048, False), (64, 64, False)))):
+        y = rng.normal(size=(m, width))
+        wide = rounded(rng.normal(size=(m, total + width)), dtype)
+        gate = wide[:, offset:offset + width]
+        g64 = gate.double().cpu().numpy()
+        for part, period, first in cases:
+            weight = rng.normal(size=period)
+            out = torch.empty(m, width, dtype=dtype, device="cuda")
+            k.gated_part_norm(torch.from_numpy(y).float().cuda(), gate, torch.from_numpy(weight).float().cuda(), out, part, 1e-5,
+                              gate_first=first, gate_kind="silu")
+            x = y.astype(np.float32).astype(np.float64)
+            if first:
+                want = P.grouped_rms_norm(x * P.silu(g64), np.tile(weight, width // period), width // part, 1e-5)
+            else:
+                want = P.grouped_rms_norm(x, np.tile(weight, width // period), width // part, 1e-5) * P.silu(g64)
+            np.testing.assert_allclose(out.double().cpu().numpy(), want, atol=tol * np.abs(want).max(), rtol=tol, err_msg=str((width, part)))
 
 
 # ---- each mixer alone in a model of one layer ------------------------------------------------------------------------
