@@ -209,6 +209,8 @@ struct SkinnyEpilogue {
     float* ss_out;            // [M][gridDim.x]
     int cols;                 // PAIR: the output columns of a workgroup, 17..32 (otherwise 16, whatever this says)
     int ss_stride;            // floats between the rows of ss_out (its capacity: a strip of 16 a part)
+    float glu_limit;          // GATED: > 0: the clamped gate g = min(gate, limit), u = clamp(up, +-limit),
+    float glu_slope;          //        y = g sigmoid(slope g) (u + 1); 0: y = silu(gate) up
 };
 
 // PAIR: a workgroup owns `cols` (17..32) output columns, two strips side by side, the second one partly
@@ -435,7 +437,15 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
                 if constexpr (EPI == EPI_SCALE) v[g] *= row_scale;
             }
             float y = v[0];
-            if (GATED) y = (v[0] / (1.0f + expf(-v[0]))) * v[NW - 1];
+            if (GATED) {
+                if (epi.glu_limit > 0.f) {
+                    const float gg = fminf(v[0], epi.glu_limit);
+                    const float uu = fminf(fmaxf(v[NW - 1], -epi.glu_limit), epi.glu_limit);
+                    y = (gg / (1.0f + expf(-epi.glu_slope * gg))) * (uu + 1.0f);
+                } else {
+                    y = (v[0] / (1.0f + expf(-v[0]))) * v[NW - 1];
+                }
+            }
             y4[i][r] = y;
             if constexpr (PAIR) y4b[r] = v[1];
             if constexpr (PAIR && EPI != EPI_RESIDUAL) {  // the second strip's sum of this lane: column n0 + 16 + 4 b + r
@@ -969,6 +979,21 @@ extern "C" int mlr_gemm_gated_silu(const void* a, const void* w, void* out, int 
     if (M <= 64) return launch_skinny<4, true>(a, w, out, M, N, K, 0, stream);
     if (K % WIDE_BK == 0 && (unsigned long long)M * K < (1ull << 31) && 2ull * N * K < (1ull << 31))
         return launch_wide_shape<true>(wide_shape_for(M, N, true), a, w, out, M, N, K, 0, stream);
+    return 1;
+}
+
+// out[M, N] = g sigmoid(slope g) (u + 1) with g = min(a . w[0:N]^T, limit), u = clamp(a . w[N:2N]^T, -limit, limit):
+// the clamped gate as the epilogue of the weight-streaming kernels, up to 64 rows.  Returns 1 for more rows.
+extern "C" int mlr_gemm_gated_clamped(const void* a, const void* w, void* out, int M, int N, int K, float limit,
+                                      float slope, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0 || !(limit > 0.f)) return -1;
+    SkinnyEpilogue epi{};
+    epi.glu_limit = limit;
+    epi.glu_slope = slope;
+    if (M <= 16) return launch_skinny<1, true>(a, w, out, M, N, K, 0, stream, epi);
+    if (M <= 32) return launch_skinny<2, true>(a, w, out, M, N, K, 0, stream, epi);
+    if (M <= 64) return launch_skinny<4, true>(a, w, out, M, N, K, 0, stream, epi);
     return 1;
 }
 

@@ -297,6 +297,21 @@ class Kernels:
         fn = self._lib("gemm").mlr_gemm_gated_silu
         _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(two_n // 2), _c_int(k), _stream()), "gemm_gated_silu")
 
+    @timed("gemm", _gemm_work)
+    def gemm_gated_clamped(self, a, w, out, limit, slope):
+        """out[M, N] = g sigmoid(slope g) (u + 1), g = min(a . w[:N]^T, limit), u = clamp(a . w[N:]^T, -limit, limit):
+        the clamped gate fused into the weight-streaming projection, up to 64 rows (bfloat16)."""
+        _need(self.dtype == torch.bfloat16 and a.shape[0] <= 64, "gemm_gated_clamped: bfloat16, up to 64 rows")
+        _tensor(a, "a", self.dtype, ndim=2)
+        _tensor(w, "w", self.dtype, ndim=2)
+        m, k = a.shape
+        two_n, k2 = w.shape
+        _need(k == k2 and two_n % 2 == 0 and limit > 0, "gemm_gated_clamped: sizes do not fit")
+        _tensor(out, "out", self.dtype, (m, two_n // 2))
+        fn = self._lib("gemm").mlr_gemm_gated_clamped
+        _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(two_n // 2), _c_int(k), _c_float(limit), _c_float(slope), _stream()),
+            "gemm_gated_clamped")
+
     # -- an RMSNorm handed from one projection to the next (few rows) ------------------------------
     HANDOFF_MAX_ROWS = 16
 

@@ -102,10 +102,13 @@ class ClampedGluMlp:
         s = self.spec
         m = x.shape[0]
         k = ctx.kernels
-        gate_up = ctx.workspace.get("gate_up", (m, 2 * s.intermediate), x.dtype)
-        k.gemm(x, self.gate_up, gate_up)
         act = ctx.workspace.get("act", (m, s.intermediate), x.dtype)
-        k.clamped_glu(gate_up, act, float(s.limit), float(s.slope))
+        if k.streams_weight(m, s.hidden):             # few rows: the activation rides on the projection
+            k.gemm_gated_clamped(x, self.gate_up, act, float(s.limit), float(s.slope))
+        else:
+            gate_up = ctx.workspace.get("gate_up", (m, 2 * s.intermediate), x.dtype)
+            k.gemm(x, self.gate_up, gate_up)
+            k.clamped_glu(gate_up, act, float(s.limit), float(s.slope))
         out = ctx.workspace.get("ffn_out", (m, s.hidden), x.dtype)
         k.gemm(act, self.down, out)
         return out

@@ -409,6 +409,21 @@ def test_row_kernels(dtype_name, width, inter):
     np.testing.assert_allclose(act.double().cpu().numpy(), want, atol=tol, rtol=tol)
 
 
+@pytest.mark.parametrize("rows", [1, 8, 17, 40, 64])
+def test_the_clamped_gate_fused_into_the_projection(rows):
+    from mini_llm_runtime_amd.kernels import Kernels
+    k = Kernels(torch.bfloat16)
+    rng = np.random.default_rng(rows)
+    n, inner = 72, 200
+    a = rounded(rng.normal(size=(rows, inner)), torch.bfloat16)
+    w = rounded(rng.normal(size=(2 * n, inner)) * 0.1, torch.bfloat16)
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device="cuda")
+    k.gemm_gated_clamped(a, w, out, 0.9, 1.702)
+    w64 = w.double().cpu().numpy()
+    want = P.clamped_glu(a.double().cpu().numpy(), {"gate": w64[:n], "up": w64[n:], "down": np.eye(n)}, dict(limit=0.9))
+    np.testing.assert_allclose(out.double().cpu().numpy(), want, atol=1e-2, rtol=1e-2)
+
+
 @pytest.mark.parametrize("dtype_name", DTYPES)
 @pytest.mark.parametrize("offset,total", [(100, 300), (96, 304)])              # the gate's columns: unaligned, aligned to 16 bytes
 def test_gated_norm_in_parts(dtype_name, offset, total):
