@@ -615,3 +615,62 @@ def test_the_command_line_runs_a_random_model(tmp_path):
     assert report["input_token_ids"] == [1, 2, 3, 4, 5] and len(report["token_ids"]) == 5
     if report["dtype"] == "float32":
         assert report["token_ids"] == want(folder).greedy([1, 2, 3, 4, 5], 5)
+
+
+def drawn_config(rng):
+    """A Taletar configuration drawn at random: any order of layers, head sizes that the matrix-core kernels take or
+    not, shared kv heads or not, one to eight taps, any grouping that divides."""
+    width = int(rng.choice([40, 64, 72, 96, 136]))
+    layers = []
+    for _ in range(int(rng.integers(1, 5))):
+        kind = rng.choice(["attention", "gla", "mamba2"])
+        if kind == "attention":
+            kv = int(rng.choice([1, 2, 3]))
+            heads = kv * int(rng.choice([1, 2, 4, 5]))
+            dim = int(rng.choice([8, 16, 20, 32, 48, 64]))
+            layer = attention(heads, kv, dim, int(rng.choice([8, 16, 24, 48, 80, 144])), diff=float(rng.uniform(0.0, 0.8)),
+                              temp=None if rng.random() < 0.25 else (float(rng.uniform(0.1, 1.0)), int(rng.choice([1, 3, 8, 50]))),
+                              cap=float(rng.choice([2.0, 10.0, 50.0])))
+            if rng.random() < 0.2:
+                del layer["mixer"]["softcap"]
+        elif kind == "gla":
+            layer = gla(int(rng.integers(1, 5)), int(rng.choice([4, 16, 24, 33, 70])), int(rng.choice([8, 20, 64, 72])),
+                        float(rng.choice([1.0, 4.0, 16.0])), int(rng.integers(1, 9)))
+        else:
+            groups = int(rng.choice([1, 2, 3]))
+            heads = groups * int(rng.choice([1, 2, 4]))
+            vdim = int(rng.choice([4, 8, 16, 40]))
+            parts = [p for p in (1, 2, 4, heads, heads * vdim) if (heads * vdim) % p == 0]
+            layer = mamba(heads, vdim, int(rng.choice([4, 16, 24, 65])), groups, int(rng.integers(1, 9)), int(rng.choice(parts)))
+        layers.append(dense(layer, None if rng.random() < 0.25 else int(rng.choice([24, 64, 100])), float(rng.uniform(0.5, 3.0))))
+    return dict(architecture="Taletar", vocab=int(rng.choice([33, 100, 257])), width=width,
+                norm=dict(eps=float(rng.choice([1e-6, 1e-5, 1e-3]))), layers=layers)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    from mini_llm_runtime_amd.config import config_from_dict
+    from mini_llm_runtime_amd.engine import Runner
+    from mini_llm_runtime_amd.parts import DecoderModel
+    from mini_llm_runtime_amd.weights import write_random_model
+    rng = np.random.default_rng(1000 + seed)
+    cfg = drawn_config(rng)
+    folder = str(tmp_path)
+    write_random_model(folder, config_from_dict(cfg), seed=seed, matrix_std=0.1, norm_std=0.2)
+    reqs = make_requests(cfg["vocab"], [90, 37, 5, 64], seed=seed)
+    want = plain_logits(P.PlainTaletar(folder), reqs)
+    scale = max(float(np.abs(v).max()) for v in want.values())
+    page = int(rng.choice([4, 8, 16, 24, 32]))
+    steps, peak = mixed(reqs, seed=seed)
+    for dtype_name in DTYPES:
+        model = DecoderModel.load(folder, DTYPES[dtype_name])
+        results = {}
+        for mode, trace, pool in (("whole", whole(reqs), 128), ("portions", portions(reqs), 128), ("mixed", steps, peak)):
+            r = Runner(model, max_tokens=pool, max_slots=4, page_size=page, max_length=256, split_keys=64)
+            results[mode] = run_steps(r, trace)
+            close(results[mode], want, dtype_name, scale, outliers=None if dtype_name == "float32" else max(2, len(want) // 25))
+            r.cache.check()
+            assert r.free_slots() == 4
+        if dtype_name == "float32":
+            assert max_difference(results["whole"], results["portions"]) == 0.0, cfg
+            assert max_difference(results["whole"], results["mixed"]) == 0.0, cfg
