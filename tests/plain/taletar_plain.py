@@ -39,9 +39,9 @@ def query_temperature(positions, coef, every):
 
 
 def capped_scores(q, k, scale, softcap):
-    """[Tq, Tk] scores of one map of one head: scaled, then squashed into (-softcap, softcap)."""
+    """[Tq, Tk] scores of one map of one head: scaled, then squashed into (-softcap, softcap) (None: no cap)."""
     s = (q @ k.T) * scale
-    return softcap * np.tanh(s / softcap)
+    return s if softcap is None else softcap * np.tanh(s / softcap)
 
 
 def causal_softmax(s, first_position=0):
@@ -71,7 +71,7 @@ def differential_attention(h, w, cfg, eps):
     heads = []
     for head in range(H):
         g = head // (H // G)
-        maps = [causal_softmax(capped_scores(q[:, head, m], k[:, g, m], cfg["scale"], cfg["softcap"])) @ v[:, g]
+        maps = [causal_softmax(capped_scores(q[:, head, m], k[:, g, m], cfg["scale"], cfg.get("softcap"))) @ v[:, g]
                 for m in range(2)]
         o = maps[0] - lam * maps[1]
         heads.append(rms_unit(o, eps) * (1.0 - cfg["diff"]))
