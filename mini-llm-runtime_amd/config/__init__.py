@@ -4,8 +4,9 @@ from .specs import (AttentionSpec, ClampedGluSpec, DiffAttentionSpec, GlaSpec, L
                     ModelSpec, NormSpec, PositionSpec, QueryTemperature)
 from .qwen3 import Qwen3Config
 from .taletar import TaletarConfig
+from .pamunex import PamunexConfig
 
 __all__ = ["ConfigError", "config_class", "config_from_dict", "known_architectures", "load_config",
            "register_architecture", "AttentionSpec", "LayerRun", "LayerSpec", "MlpSpec",
            "ModelSpec", "NormSpec", "PositionSpec", "Qwen3Config", "ClampedGluSpec", "DiffAttentionSpec", "GlaSpec",
-           "Mamba2Spec", "QueryTemperature", "TaletarConfig"]
+           "Mamba2Spec", "QueryTemperature", "TaletarConfig", "PamunexConfig"]

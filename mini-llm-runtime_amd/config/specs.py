@@ -114,6 +114,81 @@ class ClampedGluSpec:
 
 
 @dataclass(frozen=True)
+class MaskSpec:
+    """Which keys a query at position p sees besides "none after it": `window`: the last `size` positions
+    (itself and the size - 1 before it); `chunk`: the positions of its own block floor(p / size)."""
+    kind: str                 # "window" | "chunk"
+    size: int
+
+
+@dataclass(frozen=True)
+class SinkAttentionSpec:
+    """Grouped-query attention whose softmax has one more summand exp(sink[head]) in its denominator (a learned
+    number a head that stands for no key and brings no value), with query/key and value sizes of their own,
+    optional biases on the q/k/v projections, a per-head norm of q and k before the rotation, a rotation of a
+    head's first channels, and a mask rule."""
+    kind: str                 # "sink_attention"
+    hidden: int
+    q_heads: int
+    kv_heads: int
+    head_dim: int             # query/key channels of a head
+    value_dim: int
+    scale: float
+    qk_norm: Optional[NormSpec] = None
+    position: Optional[PositionSpec] = None      # `dim` of it: how many of a head's first channels turn
+    mask: Optional[MaskSpec] = None              # None: every earlier key
+    sink: bool = True
+    bias: bool = False
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose keys and values of all heads are made from one latent vector a token (normed, `rank`
+    channels) by per-head up-projections, plus one rotated key part (`rot_dim` channels) that all heads share;
+    a query head has `head_dim` plain and `rot_dim` rotated channels.  Only the latent vector and the rotated key
+    part are cached.  Softmax with a sink, and a mask rule, as `SinkAttentionSpec`."""
+    kind: str                 # "latent_attention"
+    hidden: int
+    heads: int
+    head_dim: int             # plain (unrotated) query/key channels of a head
+    rot_dim: int
+    value_dim: int
+    rank: int
+    scale: float
+    eps: float                # of the latent vector's norm
+    position: PositionSpec = None                # turns the whole rotated part: dim == rot_dim
+    mask: Optional[MaskSpec] = None
+    sink: bool = True
+
+
+@dataclass(frozen=True)
+class PlainMlpSpec:
+    """down(act(up(x))) without a gate."""
+    kind: str                 # "plain_mlp"
+    hidden: int
+    intermediate: int
+    activation: str = "relu_squared"
+
+
+@dataclass(frozen=True)
+class RoutedMlpSpec:
+    """A mixture of `experts` ungated feed-forwards of which a token uses `top`: scores sigmoid(router x); the
+    experts form `group_count` equal groups of neighbours, a group's score is the sum of its two largest scores,
+    only experts of the `group_keep` best groups can be chosen; the chosen experts' scores are their weights as
+    they are (`renormalize` False) or divided by their sum."""
+    kind: str                 # "routed_mlp"
+    hidden: int
+    intermediate: int         # of one expert
+    experts: int
+    top: int
+    group_count: int = 1
+    group_keep: int = 1
+    activation: str = "relu_squared"
+    score: str = "sigmoid"
+    renormalize: bool = False
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     kind: str                 # key in the block registry, e.g. "prenorm", "parallel"
     norm1: NormSpec
@@ -144,6 +219,7 @@ class HeadSpec:
     vocab_size: int
     hidden: int
     tied: bool = False        # no tensor of its own: the embedding's table
+    scale: float = 1.0        # factor on the logits (kind "scaled_head")
 
 
 @dataclass(frozen=True)

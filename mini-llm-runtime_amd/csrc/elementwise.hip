@@ -551,6 +551,65 @@ __global__ __launch_bounds__(256) void gated_part_norm_vec_kernel(const float* _
 }
 #endif
 
+// Layer norm of a row, y = (x - mean) / sqrt(var + eps) * weight + bias with var the mean of the squared
+// deviations (two passes over the row, 32-bit), times `out_scale`.  The row comes from `xe` (the engine's element
+// type) or from `xf` (float), whichever is not null; for output row r it is row src = rows ? rows[r] : r.
+//   acc != null: acc[src] += y (the float residual stream takes a sublayer's normed output), and with
+//     cast != null also cast[src] = T(acc[src]): the stream as the next sublayer's input;
+//   else out[r] = T(y).
+// One workgroup a row.
+__global__ __launch_bounds__(256) void layernorm_kernel(const elem_t* __restrict__ xe, const float* __restrict__ xf,
+                                                        const float* __restrict__ weight, const float* __restrict__ bias,
+                                                        const int32_t* __restrict__ rows, float* __restrict__ acc,
+                                                        elem_t* __restrict__ cast, elem_t* __restrict__ out, int width,
+                                                        float eps, float out_scale) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    const elem_t* re = xe ? xe + src * width : nullptr;
+    const float* rf = xf ? xf + src * width : nullptr;
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) sum += re ? to_float(re[i]) : rf[i];
+    const float mean = block_sum(sum, scratch) / (float)width;
+    float dev = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float d = (re ? to_float(re[i]) : rf[i]) - mean;
+        dev += d * d;
+    }
+    const float inv = 1.0f / sqrtf(block_sum(dev, scratch) / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float x = re ? to_float(re[i]) : rf[i];
+        const float y = (((x - mean) * inv) * weight[i] + (bias ? bias[i] : 0.f)) * out_scale;
+        if (acc != nullptr) {
+            const float sumh = acc[src * width + i] + y;
+            acc[src * width + i] = sumh;
+            if (cast != nullptr) cast[src * width + i] = from_float<elem_t>(sumh);
+        } else {
+            out[(size_t)r * width + i] = from_float<elem_t>(y);
+        }
+    }
+}
+
+// out = relu(x)^2, element by element (32-bit).
+__global__ void relu_squared_kernel(const elem_t* __restrict__ x, elem_t* __restrict__ out, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
+        const float r = fmaxf(to_float(x[i]), 0.f);
+        out[i] = from_float<elem_t>(r * r);
+    }
+}
+
+// out = T(h): the float residual stream as a sublayer's input.
+__global__ void cast_rows_kernel(const float* __restrict__ h, elem_t* __restrict__ out, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = from_float<elem_t>(h[i]);
+}
+
+// x *= factor (float values, logits for instance).
+__global__ void scale_float_kernel(float* __restrict__ x, float factor, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        x[i] *= factor;
+}
+
 static int grid_for(size_t count, int block) {
     size_t g = (count + block - 1) / block;
     return (int)(g > 65535 ? 65535 : (g == 0 ? 1 : g));
@@ -681,6 +740,34 @@ int mlr_gated_part_norm(const float* y, const void* gate, long gate_stride, cons
     gated_part_norm_kernel<<<(unsigned)((units + 3) / 4), 256, 0, stream>>>(y, (const elem_t*)gate, gate_stride, weight,
                                                                            (elem_t*)out, rows, width, part, period, eps,
                                                                            gate_first, gate_kind);
+    return (int)hipGetLastError();
+}
+
+int mlr_layernorm(const void* xe, const float* xf, const float* weight, const float* bias, const int32_t* rows, float* acc,
+                  void* cast, void* out, int n_out, int width, float eps, float out_scale, hipStream_t stream) {
+    if (n_out <= 0) return 0;
+    if ((xe == nullptr) == (xf == nullptr) || (acc == nullptr && out == nullptr) || (acc != nullptr && rows != nullptr))
+        return -1;
+    layernorm_kernel<<<n_out, 256, 0, stream>>>((const elem_t*)xe, xf, weight, bias, rows, acc, (elem_t*)cast,
+                                                (elem_t*)out, width, eps, out_scale);
+    return (int)hipGetLastError();
+}
+
+int mlr_relu_squared(const void* x, void* out, size_t count, hipStream_t stream) {
+    if (count == 0) return 0;
+    relu_squared_kernel<<<grid_for(count, 256), 256, 0, stream>>>((const elem_t*)x, (elem_t*)out, count);
+    return (int)hipGetLastError();
+}
+
+int mlr_cast_rows(const float* h, void* out, size_t count, hipStream_t stream) {
+    if (count == 0) return 0;
+    cast_rows_kernel<<<grid_for(count, 256), 256, 0, stream>>>(h, (elem_t*)out, count);
+    return (int)hipGetLastError();
+}
+
+int mlr_scale_float(float* x, float factor, size_t count, hipStream_t stream) {
+    if (count == 0) return 0;
+    scale_float_kernel<<<grid_for(count, 256), 256, 0, stream>>>(x, factor, count);
     return (int)hipGetLastError();
 }
 

@@ -1,0 +1,392 @@
+// Products of many small matrices in one launch, and the routing of a mixture of experts around them.
+//
+// `grouped_gemm`: out_g[r, n] = act(sum_k a_g[r, k] * w_g[n, k]) for every group g, w_g = w + g * w_group being
+// [N, K] row-major.  Two ways of saying which rows a group has:
+//   offsets == null: every group takes the rows 0 .. M - 1, group g reading a + g * a_group and writing
+//     out + g * out_group with row strides lda / ldo: one projection per head on slices of wider rows;
+//   offsets != null: group g takes the rows offsets[g] .. offsets[g + 1] - 1 of a list sorted by group (rows of
+//     out; a's row is gather[row] when gather != null): the experts of a routed feed-forward.
+// act: none, or relu(x)^2.  Every output element is one sum over k in ascending order whatever rows lie beside
+// it, so a row's result does not depend on the batch.  Accumulation is 32-bit; the bfloat16 engine multiplies on
+// the matrix cores (v_mfma_f32_16x16x32_bf16, operands staged through LDS), the float engine with plain FMAs.
+//
+// Routing (32-bit): `router_topk_kernel` (logits of one token against every expert, sigmoid, the best groups
+// of neighbouring experts, the best experts within them), `route_sort_kernel` (the chosen (token, expert) pairs
+// sorted by expert: offsets, the token of every sorted row, the sorted row of every pair),
+// `route_combine_kernel` (a token's output: the weighted sum of its experts' rows, in the order of its choices).
+#include "common.h"
+
+#define ACT_NONE 0
+#define ACT_RELU2 1
+
+struct GroupedArgs {
+    const elem_t* a; long lda; long a_group;
+    const elem_t* w; long w_group;
+    void* out; long ldo; long out_group;
+    const int32_t* offsets; const int32_t* gather;
+    int M, N, K, groups, act, out_float;
+};
+
+#define GBM 64
+#define GBN 64
+
+// Which group and which rows this workgroup serves: (group, first row, one beyond the group's last row), or
+// group < 0 when the launch has more workgroups than the groups have tiles.
+__device__ __forceinline__ void tile_of(const GroupedArgs& g, int& group, int& row0, int& row_end) {
+    if (g.offsets == nullptr) {
+        group = blockIdx.z;
+        row0 = blockIdx.y * GBM;
+        row_end = g.M;
+        return;
+    }
+    int tile = blockIdx.y;
+    group = -1;
+    for (int e = 0; e < g.groups; ++e) {
+        const int first = g.offsets[e], count = g.offsets[e + 1] - first;
+        const int tiles = (count + GBM - 1) / GBM;
+        if (tile < tiles) {
+            group = e;
+            row0 = first + tile * GBM;
+            row_end = first + count;
+            return;
+        }
+        tile -= tiles;
+    }
+}
+
+__device__ __forceinline__ float activate(float x, int act) {
+    if (act == ACT_RELU2) {
+        const float r = fmaxf(x, 0.f);
+        return r * r;
+    }
+    return x;
+}
+
+#if !MLR_BF16
+#define GBK 16
+__global__ __launch_bounds__(256) void grouped_gemm_kernel(GroupedArgs g) {
+    __shared__ float as[GBK][GBM + 4];
+    __shared__ float ws[GBK][GBN + 4];
+    int group, m0, m_end;
+    tile_of(g, group, m0, m_end);
+    if (group < 0 || m0 >= m_end) return;
+    const int t = threadIdx.x, n0 = blockIdx.x * GBN;
+    const int tx = t % 16, ty = t / 16;
+    const int lrow = t / 4, lk = (t % 4) * 4;
+    const float* a = g.a + (g.offsets ? 0 : (size_t)group * g.a_group);
+    const float* w = g.w + (size_t)group * g.w_group;
+    float* out = (float*)g.out + (g.offsets ? 0 : (size_t)group * g.out_group);
+    long arow = -1;                            // the row of a that this thread stages
+    if (m0 + lrow < m_end) arow = g.gather ? g.gather[m0 + lrow] : m0 + lrow;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int k0 = 0; k0 < g.K; k0 += GBK) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int k = k0 + lk + e, wn = n0 + lrow;
+            as[lk + e][lrow] = (arow >= 0 && k < g.K) ? a[arow * g.lda + k] : 0.f;
+            ws[lk + e][lrow] = (wn < g.N && k < g.K) ? w[(size_t)wn * g.K + k] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < GBK; ++k) {
+            float av[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = as[k][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wv[j] = ws[k][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= m_end) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n < g.N) out[(size_t)m * g.ldo + n] = activate(acc[i][j], g.act);
+        }
+    }
+}
+#else
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+#define GBK 32
+#define GLDS (GBK + 8)           // elements between staged rows: 80 bytes
+
+__device__ __forceinline__ bf16x8 load_k8(const __bf16* p, int k, int K, bool vector_ok) {
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (vector_ok && k + 8 <= K) {
+        v = *reinterpret_cast<const bf16x8*>(p + k);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (k + e < K) v[e] = p[k + e];
+    }
+    return v;
+}
+
+// Workgroup tile 64 x 64: 2 x 2 wavefronts of 2 x 2 tiles of 16 x 16.
+__global__ __launch_bounds__(256) void grouped_gemm_kernel(GroupedArgs g) {
+    __shared__ __bf16 as[GBM * GLDS];
+    __shared__ __bf16 ws[GBN * GLDS];
+    int group, m0, m_end;
+    tile_of(g, group, m0, m_end);
+    if (group < 0 || m0 >= m_end) return;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, n0 = blockIdx.x * GBN;
+    const int wm = wave >> 1, wn = wave & 1;
+    const __bf16* a = g.a + (g.offsets ? 0 : (size_t)group * g.a_group);
+    const __bf16* w = g.w + (size_t)group * g.w_group;
+    const size_t out_base = g.offsets ? 0 : (size_t)group * g.out_group;
+    // 16-byte loads where every row starts at a multiple of 16 bytes
+    const bool a_vec = (g.K % 8) == 0 && (g.lda % 8) == 0 && (g.a_group % 8) == 0 &&
+                       (reinterpret_cast<uintptr_t>(g.a) % 16) == 0;
+    const bool w_vec = (g.K % 8) == 0 && (g.w_group % 8) == 0 && (reinterpret_cast<uintptr_t>(g.w) % 16) == 0;
+    const int srow = t >> 2, skc = (t & 3) * 8;      // this thread stages 8 k of row srow of both operands
+    long arow = -1;
+    if (m0 + srow < m_end) arow = g.gather ? g.gather[m0 + srow] : m0 + srow;
+    const bool wrow_ok = n0 + srow < g.N;
+    floatx4 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int k0 = 0; k0 < g.K; k0 += GBK) {
+        *reinterpret_cast<bf16x8*>(&as[srow * GLDS + skc]) =
+            arow >= 0 ? load_k8(a + arow * g.lda, k0 + skc, g.K, a_vec) : zero;
+        *reinterpret_cast<bf16x8*>(&ws[srow * GLDS + skc]) =
+            wrow_ok ? load_k8(w + (size_t)(n0 + srow) * g.K, k0 + skc, g.K, w_vec) : zero;
+        __syncthreads();
+        bf16x8 af[2], wf[2];
+        const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            af[i] = *reinterpret_cast<const bf16x8*>(&as[((wm * 2 + i) * 16 + frag_row) * GLDS + frag_k]);
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            wf[j] = *reinterpret_cast<const bf16x8*>(&ws[((wn * 2 + j) * 16 + frag_row) * GLDS + frag_k]);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+        __syncthreads();
+    }
+    // accumulator element r of a lane: row (lane / 16) * 4 + r, column lane % 16
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = n0 + (wn * 2 + j) * 16 + (lane & 15);
+            if (n >= g.N) continue;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = m0 + (wm * 2 + i) * 16 + (lane >> 4) * 4 + r;
+                if (m >= m_end) continue;
+                const float y = activate(acc[i][j][r], g.act);
+                const size_t at = out_base + (size_t)m * g.ldo + n;
+                if (g.out_float) ((float*)g.out)[at] = y;
+                else ((__bf16*)g.out)[at] = (__bf16)y;
+            }
+        }
+    }
+}
+#endif
+
+// ---------------------------------------------------------------------------------------------------------
+#define MAX_EXPERTS 256         // 64 lanes x EXPERT_REGS
+#define EXPERT_REGS 4
+
+// The largest value among the lanes' candidates and, among equals, the lowest index; every lane gets both.
+__device__ __forceinline__ void wave_best(float& value, int& index) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(value, off, MLR_WAVE);
+        const int oi = __shfl_xor(index, off, MLR_WAVE);
+        if (ov > value || (ov == value && oi < index)) {
+            value = ov;
+            index = oi;
+        }
+    }
+}
+
+// One wavefront a token.  z[e] = x . router[e] (32-bit sums), s = sigmoid(z).  The experts form `group_count`
+// equal groups of neighbours; a group's score is the sum of its two largest s (of its only one, when a group is
+// one expert); only experts of the `group_keep` best groups stand; of those the `top` largest s are chosen
+// (ties: the lower index), ids[m][i] in descending order of s with weights[m][i] = s itself.
+__global__ __launch_bounds__(64) void router_topk_kernel(const elem_t* __restrict__ x, long ldx,
+                                                         const float* __restrict__ router, int32_t* __restrict__ ids,
+                                                         float* __restrict__ weights, int width, int experts, int top,
+                                                         int group_count, int group_keep) {
+    __shared__ float s_lds[MAX_EXPERTS];
+    __shared__ float g_lds[MAX_EXPERTS];
+    const int m = blockIdx.x, lane = threadIdx.x;
+    const elem_t* row = x + (size_t)m * ldx;
+    for (int e = 0; e < experts; ++e) {
+        float part = 0.f;
+        for (int i = lane; i < width; i += 64) part = fmaf(to_float(row[i]), router[(size_t)e * width + i], part);
+        part = wave_sum(part);
+        if (lane == 0) s_lds[e] = 1.0f / (1.0f + expf(-part));
+    }
+    __syncthreads();
+    const int per = experts / group_count;
+    for (int gidx = lane; gidx < group_count; gidx += 64) {
+        float first = -INFINITY, second = -INFINITY;
+        for (int i = 0; i < per; ++i) {
+            const float v = s_lds[gidx * per + i];
+            if (v > first) {
+                second = first;
+                first = v;
+            } else if (v > second) {
+                second = v;
+            }
+        }
+        g_lds[gidx] = per >= 2 ? first + second : first;
+    }
+    __syncthreads();
+    // the groups that stand: group_keep times the best of those left; their experts become candidates
+    float cand[EXPERT_REGS];
+#pragma unroll
+    for (int i = 0; i < EXPERT_REGS; ++i) cand[i] = -INFINITY;
+    for (int round = 0; round < group_keep; ++round) {
+        float best = -INFINITY;
+        int which = 0x7fffffff;
+        for (int gidx = lane; gidx < group_count; gidx += 64) {
+            const float v = g_lds[gidx];
+            if (v > best) {                    // (ascending indices: the lowest among equals stays)
+                best = v;
+                which = gidx;
+            }
+        }
+        wave_best(best, which);
+        if (which == 0x7fffffff) break;
+        __syncthreads();
+        if (lane == 0) g_lds[which] = -INFINITY;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < EXPERT_REGS; ++i) {
+            const int e = lane + 64 * i;
+            if (e < experts && e / per == which) cand[i] = s_lds[e];
+        }
+    }
+    for (int round = 0; round < top; ++round) {
+        float best = -INFINITY;
+        int which = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < EXPERT_REGS; ++i) {
+            const int e = lane + 64 * i;
+            if (e < experts && cand[i] > best) {
+                best = cand[i];
+                which = e;
+            }
+        }
+        wave_best(best, which);
+        if (which == 0x7fffffff) which = 0, best = 0.f;      // (fewer candidates than `top`: refused on the host)
+#pragma unroll
+        for (int i = 0; i < EXPERT_REGS; ++i)
+            if (lane + 64 * i == which) cand[i] = -INFINITY;
+        if (lane == 0) {
+            ids[(size_t)m * top + round] = which;
+            weights[(size_t)m * top + round] = best;
+        }
+    }
+}
+
+// The `pairs` chosen (token, expert) pairs sorted by expert, by ONE workgroup: offsets[e] .. offsets[e + 1] are
+// expert e's rows of the sorted list, token_of[row] the pair's token, row_of[pair] where the pair went.  The
+// order of an expert's rows among themselves is whatever the atomics give; no result depends on it.
+__global__ __launch_bounds__(1024) void route_sort_kernel(const int32_t* __restrict__ ids, int pairs, int top,
+                                                          int experts, int32_t* __restrict__ offsets,
+                                                          int32_t* __restrict__ token_of, int32_t* __restrict__ row_of) {
+    __shared__ int count[MAX_EXPERTS + 1];
+    __shared__ int cursor[MAX_EXPERTS];
+    const int t = threadIdx.x;
+    for (int e = t; e <= experts; e += blockDim.x) count[e] = 0;
+    __syncthreads();
+    for (int i = t; i < pairs; i += blockDim.x) atomicAdd(&count[ids[i]], 1);
+    __syncthreads();
+    if (t == 0) {
+        int at = 0;
+        for (int e = 0; e < experts; ++e) {
+            const int n = count[e];
+            cursor[e] = at;
+            offsets[e] = at;
+            at += n;
+        }
+        offsets[experts] = at;
+    }
+    __syncthreads();
+    for (int i = t; i < pairs; i += blockDim.x) {
+        const int row = atomicAdd(&cursor[ids[i]], 1);
+        token_of[row] = i / top;
+        row_of[i] = row;
+    }
+}
+
+// out[m, :] = sum_i weights[m][i] * y[row_of[m * top + i], :], the sum in 32-bit in the order of the choices.
+__global__ void route_combine_kernel(const elem_t* __restrict__ y, const int32_t* __restrict__ row_of,
+                                     const float* __restrict__ weights, elem_t* __restrict__ out, int width, int top) {
+    const int m = blockIdx.x;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        float sum = 0.f;
+        for (int i = 0; i < top; ++i)
+            sum = fmaf(weights[(size_t)m * top + i], to_float(y[(size_t)row_of[(size_t)m * top + i] * width + c]), sum);
+        out[(size_t)m * width + c] = from_float<elem_t>(sum);
+    }
+}
+
+extern "C" {
+
+int mlr_grouped_gemm(const void* a, long lda, long a_group, const void* w, long w_group, void* out, long ldo,
+                     long out_group, const int32_t* offsets, const int32_t* gather, int M, int N, int K, int groups,
+                     int act, int out_float, hipStream_t stream) {
+    if (M <= 0 || N <= 0 || groups <= 0) return 0;
+    if (K <= 0 || (act != ACT_NONE && act != ACT_RELU2)) return -1;
+#if !MLR_BF16
+    out_float = 1;
+#endif
+    GroupedArgs g{(const elem_t*)a, lda, a_group, (const elem_t*)w, w_group, out, ldo, out_group, offsets, gather,
+                  M, N, K, groups, act, out_float};
+    const int row_tiles = (M + GBM - 1) / GBM + (offsets ? groups : 0);
+    if (row_tiles > 65535 || groups > 65535) return -2;
+    dim3 grid((N + GBN - 1) / GBN, row_tiles, offsets ? 1 : groups);
+    grouped_gemm_kernel<<<grid, 256, 0, stream>>>(g);
+    return (int)hipGetLastError();
+}
+
+int mlr_router_topk(const void* x, long ldx, const float* router, int32_t* ids, float* weights, int rows, int width,
+                    int experts, int top, int group_count, int group_keep, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (experts < 1 || experts > MAX_EXPERTS || group_count < 1 || experts % group_count != 0 || group_keep < 1 ||
+        group_keep > group_count || top < 1 || top > group_keep * (experts / group_count))
+        return -1;
+    router_topk_kernel<<<rows, 64, 0, stream>>>((const elem_t*)x, ldx, router, ids, weights, width, experts, top,
+                                                group_count, group_keep);
+    return (int)hipGetLastError();
+}
+
+int mlr_route_sort(const int32_t* ids, int pairs, int top, int experts, int32_t* offsets, int32_t* token_of,
+                   int32_t* row_of, hipStream_t stream) {
+    if (pairs <= 0) return 0;
+    if (experts < 1 || experts > MAX_EXPERTS || top < 1) return -1;
+    route_sort_kernel<<<1, 1024, 0, stream>>>(ids, pairs, top, experts, offsets, token_of, row_of);
+    return (int)hipGetLastError();
+}
+
+int mlr_route_combine(const void* y, const int32_t* row_of, const float* weights, void* out, int rows, int width,
+                      int top, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    route_combine_kernel<<<rows, 256, 0, stream>>>((const elem_t*)y, row_of, weights, (elem_t*)out, width, top);
+    return (int)hipGetLastError();
+}
+
+}  // extern "C"

@@ -44,6 +44,8 @@ HIP_LIBRARIES = {
     "gemm": (["gemm.hip"], ["common.h"], True),
     "recurrence": (["recurrence.hip"], ["common.h"], True),
     "diff_attention": (["diff_attention.hip"], ["common.h"], True),
+    "sink_attention": (["sink_attention.hip"], ["common.h"], True),
+    "grouped_gemm": (["grouped_gemm.hip"], ["common.h"], True),
     "attention_tiles": (["attention_tiles.hip"], [], False),      # bfloat16 only by nature
     "sampling": (["sampling.hip"], ["no_alloc.h"], False),
     "library_gemm": (["library_gemm.hip"], [], False, ["-lhipblaslt"]),      # host code around hipBLASLt

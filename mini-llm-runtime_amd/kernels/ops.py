@@ -975,6 +975,251 @@ class Kernels:
                _c_float(temp_every), _c_float(lam), _c_float(out_scale), _c_float(eps), _c_int(split_keys),
                _c_int(max_splits), _c_int(max_context), _stream()), "diff_attention_tiles")
 
+    # -- layer norm, plain activations ---------------------------------------------------------
+    @timed("norm", _tensors_work())
+    def layernorm_add(self, delta, weight, bias, h, cast=None, eps=1e-5):
+        """h += layernorm(delta) * weight + bias, row by row (h the float residual stream, delta a sublayer's
+        output); `cast`, when given, receives T(h): the stream as the next sublayer's input."""
+        _tensor(h, "h", torch.float32, ndim=2)
+        m, width = h.shape
+        _tensor(delta, "delta", self.dtype, (m, width))
+        _tensor(weight, "weight", torch.float32, (width,))
+        if bias is not None:
+            _tensor(bias, "bias", torch.float32, (width,))
+        if cast is not None:
+            _tensor(cast, "cast", self.dtype, (m, width))
+        _ok(self._lib("elementwise").mlr_layernorm(_p(delta), _ptr(0), _p(weight), _p(bias), _ptr(0), _p(h), _p(cast),
+                                                   _ptr(0), _c_int(m), _c_int(width), _c_float(eps), _c_float(1.0),
+                                                   _stream()), "layernorm_add")
+
+    @timed("norm", _tensors_work())
+    def layernorm_rows(self, h, weight, bias, out, eps, rows=None, out_scale=1.0):
+        """out[r] = T((layernorm(h[rows[r] or r]) * weight + bias) * out_scale), h float."""
+        _tensor(h, "h", torch.float32, ndim=2)
+        m, width = h.shape
+        _tensor(weight, "weight", torch.float32, (width,))
+        if bias is not None:
+            _tensor(bias, "bias", torch.float32, (width,))
+        if rows is not None:
+            _tensor(rows, "rows", torch.int32, ndim=1)
+        n_out = rows.numel() if rows is not None else m
+        _tensor(out, "out", self.dtype, (n_out, width))
+        _ok(self._lib("elementwise").mlr_layernorm(_ptr(0), _p(h), _p(weight), _p(bias), _p(rows), _ptr(0), _ptr(0),
+                                                   _p(out), _c_int(n_out), _c_int(width), _c_float(eps),
+                                                   _c_float(out_scale), _stream()), "layernorm_rows")
+
+    @timed("activation", _tensors_work())
+    def relu_squared(self, x, out):
+        """out = max(x, 0)^2 (x and out may be the same tensor)."""
+        _tensor(x, "x", self.dtype)
+        _tensor(out, "out", self.dtype, tuple(x.shape))
+        _ok(self._lib("elementwise").mlr_relu_squared(_p(x), _p(out), _c_size_t(x.numel()), _stream()), "relu_squared")
+
+    @timed("norm", _tensors_work())
+    def cast_rows(self, h, out):
+        """out = T(h), h float."""
+        _tensor(h, "h", torch.float32)
+        _tensor(out, "out", self.dtype, tuple(h.shape))
+        _ok(self._lib("elementwise").mlr_cast_rows(_p(h), _p(out), _c_size_t(h.numel()), _stream()), "cast_rows")
+
+    @timed("activation", _tensors_work())
+    def scale_float(self, x, factor):
+        """x *= factor, x float."""
+        _tensor(x, "x", torch.float32)
+        _ok(self._lib("elementwise").mlr_scale_float(_p(x), _c_float(factor), _c_size_t(x.numel()), _stream()),
+            "scale_float")
+
+    # -- attention with a sink and a mask rule -------------------------------------------------
+    SINK_MASKS = {None: 0, "all": 0, "window": 1, "chunk": 2}
+    SINK_MAX_KEY_DIM = 2048
+    SINK_MAX_VALUE_DIM = 1024
+
+    def _sink_pages(self, pages, name, kv_heads, page_size, least):
+        """Row-major pages [pages, kv_heads, page, row]: the row's width (at least `least`)."""
+        _tensor(pages, name, self.dtype, ndim=4)
+        _need(pages.shape[1] == kv_heads and pages.shape[2] == page_size and pages.shape[3] >= least,
+              lambda: f"{name}: expected [pages, {kv_heads}, {page_size}, >= {least}], got {tuple(pages.shape)}")
+        return pages.shape[3]
+
+    @timed("rope_kv", _rope_work)
+    def sink_qkv_prep(self, proj, bias, q_out, k_pages, v_pages, block_table, slots, positions, q_norm_w, k_norm_w, eps,
+                      rope, q_heads, kv_heads, key_dim, value_dim, page_size, write_cache=True):
+        """From the stacked projection [rows, q_heads * key_dim + kv_heads * (key_dim + value_dim)]: bias (float, may be
+        None), per-head RMSNorm of q and k (weights may be None), rotation of a head's first rope.shape[1] channels
+        in pairs (j, j + half) (rope float [positions, rot]: cosines | sines; may be None); q to q_out, k and v into
+        their row-major pages."""
+        total = q_heads * key_dim + kv_heads * (key_dim + value_dim)
+        _tensor(proj, "proj", self.dtype, ndim=2)
+        rows = proj.shape[0]
+        _need(proj.shape[1] == total, lambda: f"proj: expected width {total}, got {proj.shape[1]}")
+        if bias is not None:
+            _tensor(bias, "bias", torch.float32, (total,))
+        _tensor(q_out, "q_out", self.dtype, (rows, q_heads * key_dim))
+        _need(1 <= key_dim <= self.SINK_MAX_KEY_DIM, f"key_dim {key_dim}: up to {self.SINK_MAX_KEY_DIM}")
+        k_row = self._sink_pages(k_pages, "k_pages", kv_heads, page_size, key_dim)
+        v_row = self._sink_pages(v_pages, "v_pages", kv_heads, page_size, value_dim)
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _tensor(positions, "positions", torch.int32, (rows,))
+        if q_norm_w is not None:
+            _tensor(q_norm_w, "q_norm_w", torch.float32, (key_dim,))
+            _tensor(k_norm_w, "k_norm_w", torch.float32, (key_dim,))
+        rot = 0
+        if rope is not None:
+            _tensor(rope, "rope", torch.float32, ndim=2)
+            rot = rope.shape[1]
+            _need(2 <= rot <= key_dim and rot % 2 == 0, f"rope: the table's width {rot} must be even and at most {key_dim}")
+        _ok(self._lib("sink_attention").mlr_sink_qkv_prep(
+            _p(proj), ctypes.c_long(total), _p(bias), _p(q_out), _p(k_pages), ctypes.c_long(k_row), _p(v_pages),
+            ctypes.c_long(v_row), _p(block_table), _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(q_norm_w),
+            _p(k_norm_w), _c_float(eps), _p(rope), _c_int(rot), _c_int(rows), _c_int(q_heads), _c_int(kv_heads),
+            _c_int(key_dim), _c_int(value_dim), _c_int(page_size), _c_int(1 if write_cache else 0), _stream()),
+            "sink_qkv_prep")
+
+    @timed("rope_kv", _rope_work)
+    def latent_prep(self, proj, q_out, pages, block_table, slots, positions, norm_w, eps, rope, heads, dim, rot, rank,
+                    page_size, write_cache=True):
+        """Latent attention's row work on proj [rows, heads * (dim + rot) + rank + rot]: every head's rotated query
+        channels turned into q_out[:, head, rank:], the latent part normed and the shared rotated key part turned
+        into the token's cache row [rank + rot] of pages [pages, 1, page, rank + rot]."""
+        _tensor(proj, "proj", self.dtype, ndim=2)
+        rows = proj.shape[0]
+        _need(proj.shape[1] == heads * (dim + rot) + rank + rot, "proj: wrong width")
+        _tensor(q_out, "q_out", self.dtype, (rows, heads * (rank + rot)))
+        _need(self._sink_pages(pages, "pages", 1, page_size, rank + rot) == rank + rot, "pages: rows of rank + rot")
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _tensor(positions, "positions", torch.int32, (rows,))
+        _tensor(norm_w, "norm_w", torch.float32, (rank,))
+        _tensor(rope, "rope", torch.float32, ndim=2)
+        _need(rope.shape[1] == rot and rot % 2 == 0 and rot >= 2, "rope: as wide as the rotated part, which is even")
+        _ok(self._lib("sink_attention").mlr_latent_prep(
+            _p(proj), ctypes.c_long(proj.shape[1]), _p(q_out), _p(pages), ctypes.c_long(rank + rot), _p(block_table),
+            _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(norm_w), _c_float(eps), _p(rope), _c_int(rows),
+            _c_int(heads), _c_int(dim), _c_int(rot), _c_int(rank), _c_int(page_size), _c_int(1 if write_cache else 0),
+            _stream()), "latent_prep")
+
+    @timed("attention")
+    def sink_attention(self, q, k_pages, v_pages, block_table, slots, positions, sink, out, q_heads, kv_heads, key_dim,
+                       value_dim, page_size, scale, mask=None, mask_size=0):
+        """out[m, h] = softmax (with one more summand exp(sink[h]) in the denominator; sink None: none) over the keys
+        that token m sees of q.k * scale, times v.  mask: None/"all" (positions <= its own), "window" (the last
+        mask_size positions), "chunk" (its own block of mask_size positions).  Keys are the first key_dim channels of
+        k_pages' rows, values the first value_dim of v_pages' rows (which may be the same tensor)."""
+        _tensor(q, "q", self.dtype, ndim=2)
+        rows = q.shape[0]
+        _need(q.shape[1] == q_heads * key_dim, "q: wrong width")
+        _need(1 <= key_dim <= self.SINK_MAX_KEY_DIM and 1 <= value_dim <= self.SINK_MAX_VALUE_DIM,
+              f"sink_attention: keys up to {self.SINK_MAX_KEY_DIM} channels, values up to {self.SINK_MAX_VALUE_DIM}")
+        _need(q_heads % kv_heads == 0 and q_heads <= 65535, "q_heads must be a multiple of kv_heads")
+        k_row = self._sink_pages(k_pages, "k_pages", kv_heads, page_size, key_dim)
+        v_row = self._sink_pages(v_pages, "v_pages", kv_heads, page_size, value_dim)
+        _need(mask in self.SINK_MASKS, f"mask {mask!r}: one of all, window, chunk")
+        kind = self.SINK_MASKS[mask]
+        _need(kind == 0 or mask_size >= 1, "a window or chunk needs a positive size")
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _tensor(positions, "positions", torch.int32, (rows,))
+        if sink is not None:
+            _tensor(sink, "sink", torch.float32, (q_heads,))
+        _tensor(out, "out", self.dtype, (rows, q_heads * value_dim))
+        _ok(self._lib("sink_attention").mlr_sink_attention(
+            _p(q), ctypes.c_long(q.shape[1]), _p(k_pages), ctypes.c_long(k_row), _p(v_pages), ctypes.c_long(v_row),
+            _p(block_table), _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(sink), _p(out),
+            ctypes.c_long(out.shape[1]), _c_int(rows), _c_int(q_heads), _c_int(kv_heads), _c_int(key_dim),
+            _c_int(value_dim), _c_int(page_size), _c_int(kind), _c_int(int(mask_size)), _c_float(scale), _stream()),
+            "sink_attention")
+
+    # -- many small products, routing ----------------------------------------------------------
+    GROUPED_ACTS = {None: 0, "relu_squared": 1}
+    MAX_EXPERTS = 256
+
+    @timed("gemm")
+    def heads_gemm(self, a, w, out, act=None):
+        """out[:, g, :] = act(a[:, g, :] . w[g]^T) for every group g: a [rows, groups, K] and out [rows, groups, N] may be
+        views into wider rows (last stride 1, one stride per group), w [groups, N, K] contiguous."""
+        for t, name in ((a, "a"), (out, "out")):
+            _need(isinstance(t, torch.Tensor) and t.is_cuda and t.dtype is self.dtype and t.dim() == 3 and t.stride(2) == 1,
+                  f"heads_gemm: {name} must be a [rows, groups, width] view of the engine's element type")
+        _tensor(w, "w", self.dtype, ndim=3)
+        rows, groups, k = a.shape
+        _need(w.shape[0] == groups and w.shape[2] == k and tuple(out.shape) == (rows, groups, w.shape[1]),
+              "heads_gemm: shapes do not fit")
+        _need(act in self.GROUPED_ACTS, f"heads_gemm: activation {act!r}")
+        n = w.shape[1]
+        _ok(self._lib("grouped_gemm").mlr_grouped_gemm(
+            _p(a), ctypes.c_long(a.stride(0)), ctypes.c_long(a.stride(1)), _p(w), ctypes.c_long(n * k), _p(out),
+            ctypes.c_long(out.stride(0)), ctypes.c_long(out.stride(1)), _ptr(0), _ptr(0), _c_int(rows), _c_int(n), _c_int(k),
+            _c_int(groups), _c_int(self.GROUPED_ACTS[act]), _c_int(0), _stream()), "heads_gemm")
+
+    @timed("gemm")
+    def experts_gemm(self, a, w, out, offsets, gather=None, act=None):
+        """Rows sorted by expert: out[r] = act(a[gather[r] or r] . w[e]^T) for offsets[e] <= r < offsets[e + 1];
+        a [*, K], w [experts, N, K], out [rows, N], offsets int32 [experts + 1] on the device."""
+        _tensor(a, "a", self.dtype, ndim=2)
+        _tensor(w, "w", self.dtype, ndim=3)
+        experts, n, k = w.shape
+        _need(a.shape[1] == k, "experts_gemm: inner sizes differ")
+        _tensor(out, "out", self.dtype, ndim=2)
+        rows = out.shape[0]
+        _need(out.shape[1] == n, "experts_gemm: out has the wrong width")
+        _tensor(offsets, "offsets", torch.int32, (experts + 1,))
+        if gather is not None:
+            _tensor(gather, "gather", torch.int32, (rows,))
+        else:
+            _need(a.shape[0] == rows, "experts_gemm: without a gather list a has out's rows")
+        _need(act in self.GROUPED_ACTS, f"experts_gemm: activation {act!r}")
+        _ok(self._lib("grouped_gemm").mlr_grouped_gemm(
+            _p(a), ctypes.c_long(k), ctypes.c_long(0), _p(w), ctypes.c_long(n * k), _p(out), ctypes.c_long(n),
+            ctypes.c_long(0), _p(offsets), _p(gather), _c_int(rows), _c_int(n), _c_int(k), _c_int(experts),
+            _c_int(self.GROUPED_ACTS[act]), _c_int(0), _stream()), "experts_gemm")
+
+    @timed("gemm")
+    def router_topk(self, x, router, ids, weights, group_count, group_keep):
+        """Per row of x [rows, width]: s = sigmoid(x . router^T) (router float [experts, width], sums 32-bit); of the
+        group_count equal groups of neighbouring experts the group_keep with the largest sum of their two best s stay;
+        ids [rows, top] int32 the experts with the largest s among those, weights [rows, top] float their s."""
+        _tensor(x, "x", self.dtype, ndim=2)
+        rows, width = x.shape
+        _tensor(router, "router", torch.float32, ndim=2)
+        experts = router.shape[0]
+        _need(router.shape[1] == width, "router: wrong width")
+        _tensor(ids, "ids", torch.int32, ndim=2)
+        top = ids.shape[1]
+        _need(ids.shape[0] == rows, "ids: one row a token")
+        _tensor(weights, "weights", torch.float32, (rows, top))
+        _need(1 <= experts <= self.MAX_EXPERTS and group_count >= 1 and experts % group_count == 0
+              and 1 <= group_keep <= group_count and 1 <= top <= group_keep * (experts // group_count),
+              "router_topk: experts up to 256 in equal groups, and no more choices than the kept groups hold")
+        _ok(self._lib("grouped_gemm").mlr_router_topk(_p(x), ctypes.c_long(width), _p(router), _p(ids), _p(weights),
+                                                      _c_int(rows), _c_int(width), _c_int(experts), _c_int(top),
+                                                      _c_int(group_count), _c_int(group_keep), _stream()), "router_topk")
+
+    @timed("gemm")
+    def route_sort(self, ids, experts, offsets, token_of, row_of):
+        """The (token, choice) pairs of ids [rows, top] sorted by expert: offsets int32 [experts + 1], token_of
+        [rows * top] the token of every sorted row, row_of [rows * top] the sorted row of every pair."""
+        _tensor(ids, "ids", torch.int32, ndim=2)
+        pairs = ids.numel()
+        _tensor(offsets, "offsets", torch.int32, (experts + 1,))
+        _tensor(token_of, "token_of", torch.int32, (pairs,))
+        _tensor(row_of, "row_of", torch.int32, (pairs,))
+        _need(1 <= experts <= self.MAX_EXPERTS, "route_sort: up to 256 experts")
+        _ok(self._lib("grouped_gemm").mlr_route_sort(_p(ids), _c_int(pairs), _c_int(ids.shape[1]), _c_int(experts),
+                                                     _p(offsets), _p(token_of), _p(row_of), _stream()), "route_sort")
+
+    @timed("activation", _tensors_work())
+    def route_combine(self, y, row_of, weights, out):
+        """out[m] = sum_i weights[m, i] * y[row_of[m * top + i]] (32-bit sums, in the order of the choices)."""
+        _tensor(weights, "weights", torch.float32, ndim=2)
+        rows, top = weights.shape
+        _tensor(y, "y", self.dtype, ndim=2)
+        _need(y.shape[0] == rows * top, "route_combine: one row of y a pair")
+        _tensor(row_of, "row_of", torch.int32, (rows * top,))
+        _tensor(out, "out", self.dtype, (rows, y.shape[1]))
+        _ok(self._lib("grouped_gemm").mlr_route_combine(_p(y), _p(row_of), _p(weights), _p(out), _c_int(rows),
+                                                        _c_int(y.shape[1]), _c_int(top), _stream()), "route_combine")
+
     # -- sampling ----------------------------------------------------------------------------
     def sample_scratch(self, rows):
         """(floats, ints) of scratch memory that `sample` needs for this many rows."""

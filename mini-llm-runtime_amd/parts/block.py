@@ -116,3 +116,56 @@ class ParallelBlock:
             return mixed                                  # (one delta: whoever norms next adds it)
         ctx.kernels.residual_add2(h, mixed, fed)
         return None
+
+
+@register_part("block", "postnorm")
+class PostNormBlock:
+    """The norms stand behind the sublayers: h += norm1(mixer(h)); h += norm2(ffn(h)).  Mixer and feed-forward read
+    the residual stream itself (in the engine's element type), and what they give is normed and added to the float
+    stream in one pass, which also leaves the stream for the next reader (`LayerNorm.add_into`).  `norm2` and `ffn`
+    may be missing (a layer without a feed-forward)."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        self.norm1 = build_part("norm", spec.norm1)
+        self.mixer = build_part("mixer", spec.mixer)
+        if (spec.ffn is None) != (spec.norm2 is None):
+            raise ValueError("a post-norm block has a feed-forward and its norm, or neither")
+        self.norm2 = build_part("norm", spec.norm2) if spec.norm2 is not None else None
+        self.ffn = build_part("ffn", spec.ffn) if spec.ffn is not None else None
+        for norm in (self.norm1, self.norm2):
+            if norm is not None and not hasattr(norm, "add_into"):
+                raise ValueError("a post-norm block needs norms that can add into the stream (`add_into`)")
+
+    def parts(self):
+        out = {"norm1": self.norm1, "mixer": self.mixer}
+        if self.ffn is not None:
+            out.update(norm2=self.norm2, ffn=self.ffn)
+        return out
+
+    def workspace_plan(self, rows, dtype, limits):
+        import torch
+        return {("stream", dtype): rows * self.norm1.size} if dtype != torch.float32 else {}
+
+    def forward(self, ctx, h, pending, cache_id, write_cache=True, next_norm=None):
+        import torch
+        from .registry import Streamed
+        k = ctx.kernels
+        narrow = ctx.dtype != torch.float32          # (the float engine's sublayers read h itself)
+        x = h
+        if narrow:
+            x = ctx.workspace.get("stream", tuple(h.shape), ctx.dtype)
+        if isinstance(pending, Streamed) and (not narrow or pending.x is x):
+            pass                                          # the block before left the stream where we read it
+        else:
+            if pending is not None and not isinstance(pending, Complete):
+                k.residual_add(h, pending)
+            if narrow:
+                k.cast_rows(h, x)
+        mixed = self.mixer.forward(ctx, x, cache_id, write_cache)
+        last = self.ffn is None
+        self.norm1.add_into(ctx, mixed, h, cast=x if narrow and not (last and next_norm is None) else None)
+        if not last:
+            fed = self.ffn.forward(ctx, x)
+            self.norm2.add_into(ctx, fed, h, cast=x if narrow and next_norm is not None else None)
+        return Streamed(x) if next_norm is not None else None

@@ -12,7 +12,7 @@ from ..config.specs import EmbedSpec, HeadSpec
 from ..weights.loader import WeightSpec
 from .registry import PartError, register_part
 
-__all__ = ["TokenEmbedding", "LinearHead", "EmbedSpec", "HeadSpec"]
+__all__ = ["TokenEmbedding", "LinearHead", "ScaledHead", "EmbedSpec", "HeadSpec"]
 
 
 @register_part("embed", "token_embedding")
@@ -80,4 +80,18 @@ class LinearHead:
         """float logits [R, V] of the normed rows `final` [R, E]."""
         logits = ctx.workspace.get("logits", (final.shape[0], self.spec.vocab_size), torch.float32)
         ctx.kernels.gemm(final, self.weight, logits)
+        return logits
+
+
+@register_part("head", "scaled_head")
+class ScaledHead(LinearHead):
+    """logits = (final . weight^T) * scale, the factor applied to the 32-bit logits."""
+
+    def libraries(self):
+        return ["gemm", "elementwise"]
+
+    def forward(self, ctx, final):
+        logits = super().forward(ctx, final)
+        if self.spec.scale != 1.0:
+            ctx.kernels.scale_float(logits, float(self.spec.scale))
         return logits

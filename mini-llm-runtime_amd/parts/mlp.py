@@ -112,3 +112,43 @@ class ClampedGluMlp:
         out = ctx.workspace.get("ffn_out", (m, s.hidden), x.dtype)
         k.gemm(act, self.down, out)
         return out
+
+
+ACTIVATIONS = ("relu_squared",)
+
+
+@register_part("ffn", "plain_mlp")
+class PlainMlp:
+    """down(act(up(x))) without a gate; act = relu(x)^2."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        if spec.activation not in ACTIVATIONS:
+            raise PartError(f"activation {spec.activation!r} is not built ({', '.join(ACTIVATIONS)})")
+        self.spec = spec
+        self.up = self.down = None
+
+    def weight_specs(self):
+        s = self.spec
+        return {"up": WeightSpec((s.intermediate, s.hidden)), "down": WeightSpec((s.hidden, s.intermediate))}
+
+    def bind(self, weights):
+        self.up, self.down = weights["up"], weights["down"]
+
+    def libraries(self):
+        return ["gemm", "elementwise"]
+
+    def workspace_plan(self, rows, dtype, limits):
+        s = self.spec
+        return {("act", dtype): rows * s.intermediate, ("ffn_out", dtype): rows * s.hidden}
+
+    def forward(self, ctx, x):
+        s = self.spec
+        m = x.shape[0]
+        k = ctx.kernels
+        act = ctx.workspace.get("act", (m, s.intermediate), x.dtype)
+        k.gemm(x, self.up, act)
+        k.relu_squared(act, act)
+        out = ctx.workspace.get("ffn_out", (m, s.hidden), x.dtype)
+        k.gemm(act, self.down, out)
+        return out

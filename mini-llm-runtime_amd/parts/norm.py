@@ -39,3 +39,36 @@ class RmsNorm:
     def forward(self, ctx, h, delta, out, rows=None, write_h=True):
         ctx.kernels.add_rmsnorm(h, delta, self.weight, out, self.eps, rows=rows, write_h=write_h)
         return out
+
+
+@register_part("norm", "layernorm")
+class LayerNorm:
+    """y = (x - mean) / sqrt(var + eps) * weight + bias, var the mean of the squared deviations; 32-bit."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        self.size, self.eps = spec.size, float(spec.eps)
+        self.weight = self.bias = None
+
+    def weight_specs(self):
+        return {"weight": WeightSpec((self.size,), keep_float32=True),
+                "bias": WeightSpec((self.size,), keep_float32=True, init=("normal", 0.0, 0.1))}
+
+    def bind(self, weights):
+        self.weight, self.bias = weights["weight"], weights["bias"]
+
+    def libraries(self):
+        return ["elementwise"]
+
+    def forward(self, ctx, h, delta, out, rows=None, write_h=True, out_scale=1.0):
+        """The norm of the residual stream itself (a model's final norm): x = h + delta (delta may be None; it is
+        added into h), out[r] = norm(x[rows[r] or r])."""
+        if delta is not None:
+            ctx.kernels.residual_add(h, delta)
+        ctx.kernels.layernorm_rows(h, self.weight, self.bias, out, self.eps, rows=rows, out_scale=out_scale)
+        return out
+
+    def add_into(self, ctx, delta, h, cast=None):
+        """h += norm(delta): the norm of what a sublayer gave, added to the float residual stream in the same pass;
+        `cast` (the engine's element type) receives the new h as the next sublayer's input."""
+        ctx.kernels.layernorm_add(delta, self.weight, self.bias, h, cast=cast, eps=self.eps)

@@ -103,6 +103,12 @@ class Handoff(Complete):
     ss: object
 
 
+@dataclass
+class Streamed(Complete):
+    """h is complete and `x` holds it in the engine's element type (for sublayers that read the stream itself)."""
+    x: object
+
+
 class PartError(ValueError):
     pass
 

@@ -1,0 +1,78 @@
+"""A mixture of experts with group-limited routing.  Every token scores all experts, s = sigmoid(router . x) in
+32-bit; the experts form equal groups of neighbours, a group's score is the sum of its two largest s, and only
+experts of the best groups can be chosen; of those the `top` largest s win and weigh their experts' outputs (as
+they are, or divided by their sum).  An expert is an ungated feed-forward down(act(up(x))).
+
+The step's (token, expert) pairs are sorted by expert on the device, so that every expert's rows lie side by side
+and ONE launch multiplies all of them with their own weights (`Kernels.experts_gemm`, the rows of the first product
+gathered through the sorted list); nothing of it is read on the host, so a step can be captured."""
+from __future__ import annotations
+
+import torch
+
+from ..weights.loader import WeightSpec, stacked
+from .mlp import ACTIVATIONS
+from .registry import PartError, register_part
+
+
+@register_part("ffn", "routed_mlp")
+class RoutedMlp:
+    graph_safe = True
+
+    def __init__(self, spec):
+        s = self.spec = spec
+        if s.activation not in ACTIVATIONS:
+            raise PartError(f"activation {s.activation!r} is not built ({', '.join(ACTIVATIONS)})")
+        if s.score != "sigmoid" or s.renormalize:
+            raise PartError("routing: sigmoid scores used as they are is what is built")
+        if s.experts % s.group_count != 0 or not 1 <= s.group_keep <= s.group_count or \
+                not 1 <= s.top <= s.group_keep * (s.experts // s.group_count):
+            raise PartError(f"routing: {s.experts} experts in {s.group_count} groups of which {s.group_keep} stay cannot "
+                            f"give {s.top} choices")
+        self.router = self.up = self.down = None
+
+    def weight_specs(self):
+        s = self.spec
+        specs = {"router": WeightSpec((s.experts, s.hidden), keep_float32=True, init=("normal", 0.0, 0.05))}
+        for e in range(s.experts):
+            specs[f"e{e}.up"] = WeightSpec((s.intermediate, s.hidden), stack="up")
+        for e in range(s.experts):
+            specs[f"e{e}.down"] = WeightSpec((s.hidden, s.intermediate), stack="down")
+        return specs
+
+    def bind(self, weights):
+        s = self.spec
+        self.router = weights["router"]
+        self.up = stacked([weights[f"e{e}.up"] for e in range(s.experts)]).view(s.experts, s.intermediate, s.hidden)
+        self.down = stacked([weights[f"e{e}.down"] for e in range(s.experts)]).view(s.experts, s.hidden, s.intermediate)
+
+    def libraries(self):
+        return ["grouped_gemm"]
+
+    def workspace_plan(self, rows, dtype, limits):
+        s = self.spec
+        pairs = rows * s.top
+        return {("route_ids", torch.int32): pairs, ("route_weights", torch.float32): pairs,
+                ("route_offsets", torch.int32): s.experts + 1, ("route_token", torch.int32): pairs,
+                ("route_row", torch.int32): pairs, ("route_act", dtype): pairs * s.intermediate,
+                ("route_y", dtype): pairs * s.hidden, ("ffn_out", dtype): rows * s.hidden}
+
+    def forward(self, ctx, x):
+        s = self.spec
+        m = x.shape[0]
+        k, ws = ctx.kernels, ctx.workspace
+        pairs = m * s.top
+        ids = ws.get("route_ids", (m, s.top), torch.int32)
+        weights = ws.get("route_weights", (m, s.top), torch.float32)
+        offsets = ws.get("route_offsets", (s.experts + 1,), torch.int32)
+        token_of = ws.get("route_token", (pairs,), torch.int32)
+        row_of = ws.get("route_row", (pairs,), torch.int32)
+        k.router_topk(x, self.router, ids, weights, s.group_count, s.group_keep)
+        k.route_sort(ids, s.experts, offsets, token_of, row_of)
+        act = ws.get("route_act", (pairs, s.intermediate), x.dtype)
+        k.experts_gemm(x, self.up, act, offsets, gather=token_of, act=s.activation)
+        y = ws.get("route_y", (pairs, s.hidden), x.dtype)
+        k.experts_gemm(act, self.down, y, offsets)
+        out = ws.get("ffn_out", (m, s.hidden), x.dtype)
+        k.route_combine(y, row_of, weights, out)
+        return out

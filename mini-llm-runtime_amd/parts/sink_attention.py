@@ -1,0 +1,190 @@
+"""Two mixers whose softmax has a sink -- one more summand exp(sink[head]) in the denominator, a learned number a
+head that stands for no key and brings no value -- and whose queries see the keys that a mask rule names: the last
+`size` positions (`window`) or the positions of the query's own block of `size` (`chunk`), counted from the
+request's first token.
+
+`SinkAttention`: grouped-query attention with query/key and value sizes of their own, optional biases on q, k, v,
+a norm per head of q and k before the rotation, and a rotation of a head's first channels (how many, and the
+angles, are the position part's).  Per token the cache keeps keys [kv_heads, head_dim] and values
+[kv_heads, value_dim], both row-major.
+
+`LatentAttention`: keys and values of all heads are up-projections of ONE normed latent vector a token, plus one
+rotated key part that all heads share; only the latent vector and that part are cached, [rank + rot_dim] a token.
+The up-projections are moved to the query's side: q_lat[h] = W_uk[h]^T q_plain[h], so a head's score is
+q_lat[h] . latent + q_rot[h] . k_rot -- attention of all heads over ONE shared key row whose first `rank` channels
+are also the value -- and the head's output is W_uv[h] applied to the attention's latent result.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache.manager import PAGE, PagedSpec
+from ..weights.loader import WeightSpec, stacked
+from .registry import PartError, build_part, register_part
+
+
+def _mask_of(spec):
+    if spec.mask is None:
+        return None, 0
+    if spec.mask.kind not in ("window", "chunk") or spec.mask.size < 1:
+        raise PartError(f"mask {spec.mask.kind!r} of size {spec.mask.size}: window or chunk, of a positive size")
+    return spec.mask.kind, int(spec.mask.size)
+
+
+def _rope_table(position, ctx, device, rot_limit):
+    if position is None:
+        return None
+    rotation = position.rotation(ctx.max_positions, device)
+    if rotation is None:
+        return None
+    if rotation.interleaved or rotation.dim % 2 != 0 or not 2 <= rotation.dim <= rot_limit or \
+            rotation.table.shape[1] != rotation.dim:
+        raise PartError(f"the position part turns {rotation.dim} channels: must be even, in split-half pairs, at most "
+                        f"{rot_limit}")
+    return rotation.table
+
+
+@register_part("mixer", "sink_attention")
+class SinkAttention:
+    graph_safe = True
+
+    def __init__(self, spec):
+        s = self.spec = spec
+        if s.q_heads % s.kv_heads != 0:
+            raise PartError(f"q_heads {s.q_heads} is no multiple of kv_heads {s.kv_heads}")
+        self.mask, self.mask_size = _mask_of(s)
+        if s.qk_norm is not None and s.qk_norm.size != s.head_dim:
+            raise PartError("the q/k norm must span one head")
+        self.position = build_part("position", s.position) if s.position is not None else None
+        self.q_width, self.k_width, self.v_width = s.q_heads * s.head_dim, s.kv_heads * s.head_dim, s.kv_heads * s.value_dim
+        self.o_width = s.q_heads * s.value_dim
+        self.qkv = self.o = self.bias = self.q_norm = self.k_norm = self.sink = None
+
+    def weight_specs(self):
+        s = self.spec
+        specs = {"q": WeightSpec((self.q_width, s.hidden), stack="qkv"), "k": WeightSpec((self.k_width, s.hidden), stack="qkv"),
+                 "v": WeightSpec((self.v_width, s.hidden), stack="qkv"), "o": WeightSpec((s.hidden, self.o_width))}
+        if s.bias:
+            for name, width in (("q.b", self.q_width), ("k.b", self.k_width), ("v.b", self.v_width)):
+                specs[name] = WeightSpec((width,), keep_float32=True, init=("normal", 0.0, 0.02))
+        if s.qk_norm is not None:
+            specs["q.norm"] = WeightSpec((s.head_dim,), keep_float32=True)
+            specs["k.norm"] = WeightSpec((s.head_dim,), keep_float32=True)
+        if s.sink:
+            specs["sink"] = WeightSpec((s.q_heads,), keep_float32=True, init=("normal", 0.0, 1.0))
+        return specs
+
+    def bind(self, weights):
+        s = self.spec
+        self.qkv = stacked([weights["q"], weights["k"], weights["v"]])
+        self.o = weights["o"]
+        self.bias = torch.cat([weights["q.b"], weights["k.b"], weights["v.b"]]).contiguous() if s.bias else None
+        if s.qk_norm is not None:
+            self.q_norm, self.k_norm = weights["q.norm"], weights["k.norm"]
+        self.sink = weights["sink"] if s.sink else None
+
+    def cache_spec(self):
+        s = self.spec
+        return PagedSpec((("k", (s.kv_heads, PAGE, s.head_dim)), ("v", (s.kv_heads, PAGE, s.value_dim))),
+                         self.mask_size if self.mask is not None else None)
+
+    def libraries(self):
+        return ["gemm", "sink_attention"]
+
+    def workspace_plan(self, rows, dtype, limits):
+        s = self.spec
+        return {("sink_proj", dtype): rows * (self.q_width + self.k_width + self.v_width), ("q", dtype): rows * self.q_width,
+                ("attn", dtype): rows * self.o_width, ("mixer_out", dtype): rows * s.hidden}
+
+    def forward(self, ctx, x, cache_id, write_cache=True):
+        s = self.spec
+        k = ctx.kernels
+        m = x.shape[0]
+        proj = ctx.workspace.get("sink_proj", (m, self.qkv.shape[0]), x.dtype)
+        k.gemm(x, self.qkv, proj)
+        view = ctx.cache.paged_view(cache_id)
+        k_pages, v_pages = view.tensors["k"], view.tensors["v"]
+        q = ctx.workspace.get("q", (m, self.q_width), x.dtype)
+        rope = _rope_table(self.position, ctx, x.device, s.head_dim)
+        k.sink_qkv_prep(proj, self.bias, q, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, self.q_norm,
+                        self.k_norm, s.qk_norm.eps if s.qk_norm is not None else 0.0, rope, s.q_heads, s.kv_heads,
+                        s.head_dim, s.value_dim, view.page_size, write_cache)
+        attn = ctx.workspace.get("attn", (m, self.o_width), x.dtype)
+        k.sink_attention(q, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, self.sink, attn, s.q_heads,
+                         s.kv_heads, s.head_dim, s.value_dim, view.page_size, float(s.scale), self.mask, self.mask_size)
+        out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
+        k.gemm(attn, self.o, out)
+        return out
+
+
+@register_part("mixer", "latent_attention")
+class LatentAttention:
+    graph_safe = True
+
+    def __init__(self, spec):
+        s = self.spec = spec
+        self.mask, self.mask_size = _mask_of(s)
+        if s.position is None or s.position.dim != s.rot_dim or s.rot_dim % 2 != 0:
+            raise PartError("latent attention turns its whole rotated part: an even rot_dim with a position part as wide")
+        self.position = build_part("position", s.position)
+        self.q_width = s.heads * (s.head_dim + s.rot_dim)
+        self.row = s.rank + s.rot_dim                    # a token's cache row, and a query head after the move
+        self.o_width = s.heads * s.value_dim
+        self.proj = self.o = self.norm = self.uk_t = self.uv = self.sink = None
+
+    def weight_specs(self):
+        s = self.spec
+        specs = {"q": WeightSpec((self.q_width, s.hidden), stack="down"), "dkv": WeightSpec((self.row, s.hidden), stack="down"),
+                 "dkv.norm": WeightSpec((s.rank,), keep_float32=True),
+                 "uk": WeightSpec((s.heads * s.head_dim, s.rank)), "uv": WeightSpec((self.o_width, s.rank)),
+                 "o": WeightSpec((s.hidden, self.o_width))}
+        if s.sink:
+            specs["sink"] = WeightSpec((s.heads,), keep_float32=True, init=("normal", 0.0, 1.0))
+        return specs
+
+    def bind(self, weights):
+        s = self.spec
+        self.proj = stacked([weights["q"], weights["dkv"]])
+        self.norm = weights["dkv.norm"]
+        # the key up-projection as the queries meet it: per head [rank, head_dim]
+        self.uk_t = weights["uk"].view(s.heads, s.head_dim, s.rank).transpose(1, 2).contiguous()
+        self.uv = weights["uv"].view(s.heads, s.value_dim, s.rank)
+        self.o = weights["o"]
+        self.sink = weights["sink"] if s.sink else None
+
+    def cache_spec(self):
+        return PagedSpec((("latent", (1, PAGE, self.row)),), self.mask_size if self.mask is not None else None)
+
+    def libraries(self):
+        return ["gemm", "grouped_gemm", "sink_attention"]
+
+    def workspace_plan(self, rows, dtype, limits):
+        s = self.spec
+        return {("latent_proj", dtype): rows * (self.q_width + self.row), ("latent_q", dtype): rows * s.heads * self.row,
+                ("latent_out", dtype): rows * s.heads * s.rank, ("attn", dtype): rows * self.o_width,
+                ("mixer_out", dtype): rows * s.hidden}
+
+    def forward(self, ctx, x, cache_id, write_cache=True):
+        s = self.spec
+        k = ctx.kernels
+        m = x.shape[0]
+        ld = self.q_width + self.row
+        proj = ctx.workspace.get("latent_proj", (m, ld), x.dtype)
+        k.gemm(x, self.proj, proj)
+        view = ctx.cache.paged_view(cache_id)
+        pages = view.tensors["latent"]
+        q = ctx.workspace.get("latent_q", (m, s.heads * self.row), x.dtype)
+        rope = _rope_table(self.position, ctx, x.device, s.rot_dim)
+        k.latent_prep(proj, q, pages, view.block_table, ctx.slots, ctx.positions, self.norm, float(s.eps), rope, s.heads,
+                      s.head_dim, s.rot_dim, s.rank, view.page_size, write_cache)
+        # the plain query channels through the key up-projection, head by head, into the first `rank` channels
+        k.heads_gemm(torch.as_strided(proj, (m, s.heads, s.head_dim), (ld, s.head_dim + s.rot_dim, 1)), self.uk_t,
+                     torch.as_strided(q, (m, s.heads, s.rank), (s.heads * self.row, self.row, 1)))
+        lat = ctx.workspace.get("latent_out", (m, s.heads * s.rank), x.dtype)
+        k.sink_attention(q, pages, pages, view.block_table, ctx.slots, ctx.positions, self.sink, lat, s.heads, 1, self.row,
+                         s.rank, view.page_size, float(s.scale), self.mask, self.mask_size)
+        attn = ctx.workspace.get("attn", (m, self.o_width), x.dtype)
+        k.heads_gemm(lat.view(m, s.heads, s.rank), self.uv, attn.view(m, s.heads, s.value_dim))
+        out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
+        k.gemm(attn, self.o, out)
+        return out
