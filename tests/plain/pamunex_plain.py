@@ -130,6 +130,29 @@ def route(x, w, router):
     return chosen, np.take_along_axis(s, chosen, axis=1)
 
 
+def route_margin(x, w, router, rounding=2.0 ** -8):
+    """[T]: how far each token's choice is from another one, in units of what rounding x to `rounding` (relative,
+    per element) may move a score: the smaller of the gap between the last group kept and the first one dropped and
+    the gap between the last expert chosen and the best one left (infinite where nothing is left out), over the
+    largest such move among the token's scores.  A test that compares a rounded engine with this file may not rest
+    on tokens whose margin is a small number."""
+    n, top = router["experts"], router["top"]
+    count, keep = router["groups"]["count"], router["groups"]["keep"]
+    s = 1.0 / (1.0 + np.exp(-(x @ w["router"].T)))
+    moved = (s * (1.0 - s) * rounding * np.sqrt((x * x) @ (w["router"] ** 2).T)).max(axis=1) + 1e-300
+    per = n // count
+    blocks = s.reshape(-1, count, per)
+    best_two = np.sort(blocks, axis=2)[:, :, -2:].sum(axis=2) if per >= 2 else blocks.sum(axis=2)
+    ranked = -np.sort(-best_two, axis=1)
+    group_gap = ranked[:, keep - 1] - ranked[:, keep] if keep < count else np.full(s.shape[0], np.inf)
+    order = np.argsort(-best_two, axis=1, kind="stable")[:, :keep]
+    allowed = np.zeros((s.shape[0], count), dtype=bool)
+    np.put_along_axis(allowed, order, True, axis=1)
+    masked = -np.sort(-np.where(np.repeat(allowed, per, axis=1), s, -np.inf), axis=1)
+    expert_gap = masked[:, top - 1] - masked[:, top] if top < keep * per else np.full(s.shape[0], np.inf)
+    return np.minimum(group_gap, expert_gap) / moved
+
+
 def moe_ffn(x, w, cfg):
     chosen, weights = route(x, w, cfg["router"])
     out = np.zeros_like(x)
@@ -151,9 +174,10 @@ def layer_weights(weights, layer, part):
     return {name[len(prefix):]: value for name, value in weights.items() if name.startswith(prefix)}
 
 
-def forward(config, weights, tokens, streams=None):
+def forward(config, weights, tokens, streams=None, margins=None):
     """Logits [T, vocab] of one sequence from position 0.  `weights`: {tensor name: float64 array}.
-    `streams`, a list, receives the residual stream after every layer."""
+    `streams`, a list, receives the residual stream after every layer; `margins`, a list, the routing margin
+    [T] of every layer that routes."""
     eps = config["norm"]["eps"]
     x = weights["embed"][np.asarray(tokens)]
     for i, layer in enumerate(config["layers"]):
@@ -161,8 +185,58 @@ def forward(config, weights, tokens, streams=None):
         x = x + layer_norm(mixed, weights[f"l{i}.norm1"], weights[f"l{i}.norm1.b"], eps)
         if layer.get("mlp") is not None:
             fed = feed_forward(x, layer_weights(weights, i, "mlp"), layer["mlp"])
+            if margins is not None and layer["mlp"]["kind"] == "moe":
+                margins.append(route_margin(x, layer_weights(weights, i, "mlp"), layer["mlp"]["router"]))
             x = x + layer_norm(fed, weights[f"l{i}.norm2"], weights[f"l{i}.norm2.b"], eps)
         if streams is not None:
             streams.append(x.copy())
     x = layer_norm(x, weights["final.norm"], weights["final.norm.b"], eps)
     return (x @ weights["embed"].T) * config["logit_scale"]
+
+
+class PlainPamunex:
+    """A model folder (config.json, model.safetensors) run by the functions above."""
+
+    def __init__(self, folder):
+        import json
+        import os
+
+        import torch
+        from safetensors.torch import load_file
+        with open(os.path.join(folder, "config.json")) as f:
+            self.cfg = json.load(f)
+        self.tensors = {n: (t.to(torch.float64) if t.dtype.is_floating_point else t).numpy()
+                        for n, t in load_file(os.path.join(folder, "model.safetensors")).items()}
+
+    def logits(self, tokens, want=None):
+        rows = forward(self.cfg, self.tensors, tokens)
+        return rows if want is None else rows[np.asarray(want, dtype=np.int64)]
+
+    def routing_margins(self, tokens):
+        """[T]: the smallest routing margin of every position over the layers that route (see `route_margin`);
+        None for a model that routes nowhere."""
+        margins = []
+        forward(self.cfg, self.tensors, tokens, margins=margins)
+        return np.min(margins, axis=0) if margins else None
+
+    def decisive(self, tokens, rng, least=40.0, tries=2000):
+        """`tokens` with the token at every position whose routing is a close call (a margin below `least`) drawn
+        again, from left to right (a position's margins depend on the tokens up to it only), so that an engine that
+        rounds chooses the experts this file chooses: no comparison then rests on a close call."""
+        tokens = list(tokens)
+        vocab = self.tensors["embed"].shape[0]
+        for _ in range(tries):
+            margins = self.routing_margins(tokens)
+            near = [] if margins is None else np.nonzero(margins < least)[0]
+            if len(near) == 0:
+                return tokens
+            tokens[int(near[0])] = int(rng.integers(0, vocab))
+        raise ValueError("no decisive sequence found")
+
+    def greedy(self, prompt, n):
+        tokens, out = list(prompt), []
+        for _ in range(n):
+            t = int(np.argmax(self.logits(tokens, [len(tokens) - 1])[0]))
+            out.append(t)
+            tokens.append(t)
+        return out
