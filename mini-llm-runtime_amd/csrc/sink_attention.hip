@@ -239,6 +239,220 @@ __global__ __launch_bounds__(64) void latent_prep_kernel(
     }
 }
 
+#if MLR_BF16
+// ---------------------------------------------------------------------------------------------------------
+// The same attention on the matrix cores (bfloat16 engine; keys in multiples of 8 channels up to 576, values in
+// multiples of 16 up to 512): prompt portions and single tokens.
+//
+// A workgroup (4 wavefronts) serves ONE group of consecutive tokens of a request and up to `head_block` query heads
+// of one kv head: 64 columns (token, head), token = column / head_block.  It walks the keys that its tokens see,
+// from the first key of the group's first token to the last token's own position, in tiles of 32 keys at absolute
+// multiples of 32; a tile's key rows are staged once through LDS for all its columns (row-major for the scores,
+// and the value channels transposed, [channel][key], for the second product: 16-byte reads of eight keys of one
+// channel), the next tile's rows on their way from memory into registers meanwhile.  Where the value rows ARE the
+// key rows they are read once.  Rows outside the range, or without a page, are staged as zeros.
+//   S^T = K Q^T with v_mfma_f32_16x16x32_bf16: row i of the instruction's first operand is tile key
+//   8 (i / 4) + 4 s + i % 4 of half-tile s, so that a lane ends up with the scores of the eight CONSECUTIVE keys
+//   8 b .. 8 b + 7 (b = lane / 16) of its column (lane % 16): the probabilities are the second product's operand
+//   as they lie.  Softmax per column in 32-bit, base 2, the running maximum and sum kept by the column's four lanes.
+// SPLITV (groups of at most 16 columns: single tokens): all four wavefronts compute the same scores and each takes
+// a quarter of the value channels, so a lone token's workgroup still uses its four matrix units.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+#define TK 32                   // keys in a tile
+#define VT_PITCH 40             // elements between the channels of the transposed values (80 bytes)
+
+template <int NKF, int NVT, bool SPLITV>
+__global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, const int32_t* __restrict__ group_first,
+                                                                   const int32_t* __restrict__ group_count,
+                                                                   int head_block, int head_blocks) {
+    constexpr int KD = NKF * 32, KP = KD + 8, CPK = NKF * 4;          // padded key channels, row pitch, 16-byte chunks a key
+    constexpr int NSK = (TK * CPK + 255) / 256;                        // chunks of key rows a thread stages
+    constexpr int CPV = NVT * 2, NSV = (TK * CPV + 255) / 256;         // the same for value rows of their own
+    constexpr int NACC = SPLITV ? NVT / 4 : NVT;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    __bf16* k_lds = reinterpret_cast<__bf16*>(lds_raw);               // [TK][KP]
+    __bf16* vt_lds = k_lds + TK * KP;                                  // [NVT * 16][VT_PITCH]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int group = blockIdx.x, kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+    const int first = group_first[group], count = group_count[group];
+    const int hg = a.q_heads / a.kv_heads;
+    const int D = a.key_dim, V = a.value_dim;
+    const bool shared_rows = a.v_pages == a.k_pages;
+    const int p0 = a.positions[first], slot = a.slots[first];
+    const int kbegin = first_seen(p0, a.mask_kind, a.mask_size), kend = p0 + count;
+    const int32_t* table = a.block_table + (size_t)slot * a.max_blocks;
+
+    // this lane's column
+    const int col = (SPLITV ? 0 : wave * 16) + (lane & 15), b = lane >> 4;
+    const int ti = col / head_block, hi = hb * head_block + col % head_block;
+    const bool col_ok = ti < count && hi < hg;
+    const int head = kvh * hg + (hi < hg ? hi : 0);
+    const int m = first + (ti < count ? ti : 0);
+    const int qpos = p0 + ti;
+    const int qlo = first_seen(qpos, a.mask_kind, a.mask_size);
+    bf16x8 qf[NKF];
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int kf = 0; kf < NKF; ++kf) {
+        const int d = kf * 32 + b * 8;
+        qf[kf] = (col_ok && d < D) ? *reinterpret_cast<const bf16x8*>(a.q + (size_t)m * a.q_stride + (size_t)head * D + d) : zero8;
+    }
+    floatx4 acc[NACC];
+#pragma unroll
+    for (int j = 0; j < NACC; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    float run_max = -INFINITY, run_sum = 0.f;
+    const float scale2 = a.scale * 1.4426950408889634f;
+
+    bf16x8 kreg[NSK], vreg[NSV];
+    auto row_of_key = [&](int kp) -> long long {
+        if (kp < kbegin || kp >= kend) return -1;
+        const int block = kp / a.page_size;
+        const int page = block < a.max_blocks ? table[block] : -1;
+        return page < 0 ? -1 : ((long long)page * a.kv_heads + kvh) * a.page_size + kp % a.page_size;
+    };
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int i = 0; i < NSK; ++i) {
+            const int q = tid + 256 * i, key = q / CPK, d = (q % CPK) * 8;
+            kreg[i] = zero8;
+            if (q < TK * CPK && d < D) {
+                const long long r = row_of_key(t0 + key);
+                if (r >= 0) kreg[i] = *reinterpret_cast<const bf16x8*>(a.k_pages + r * a.k_row + d);
+            }
+        }
+        if (!shared_rows) {
+#pragma unroll
+            for (int i = 0; i < NSV; ++i) {
+                const int q = tid + 256 * i, key = q / CPV, d = (q % CPV) * 8;
+                vreg[i] = zero8;
+                if (q < TK * CPV && d < V) {
+                    const long long r = row_of_key(t0 + key);
+                    if (r >= 0) vreg[i] = *reinterpret_cast<const bf16x8*>(a.v_pages + r * a.v_row + d);
+                }
+            }
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < NSK; ++i) {
+            const int q = tid + 256 * i, key = q / CPK, d = (q % CPK) * 8;
+            if (q < TK * CPK) {
+                *reinterpret_cast<bf16x8*>(&k_lds[key * KP + d]) = kreg[i];
+                if (shared_rows && d < NVT * 16) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) vt_lds[(d + e) * VT_PITCH + key] = (d + e < V) ? kreg[i][e] : (__bf16)0.f;
+                }
+            }
+        }
+        if (!shared_rows) {
+#pragma unroll
+            for (int i = 0; i < NSV; ++i) {
+                const int q = tid + 256 * i, key = q / CPV, d = (q % CPV) * 8;
+                if (q < TK * CPV) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) vt_lds[(d + e) * VT_PITCH + key] = vreg[i][e];
+                }
+            }
+        }
+    };
+
+    const int t_first = (kbegin / TK) * TK;
+    fetch(t_first);
+    for (int t0 = t_first; t0 < kend; t0 += TK) {
+        stage();
+        __syncthreads();
+        if (t0 + TK < kend) fetch(t0 + TK);
+        // scores of this lane's column against the tile's keys 8 b .. 8 b + 7
+        floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+        const int i16 = lane & 15;
+        const int krow0 = 8 * (i16 >> 2) + (i16 & 3);
+#pragma unroll
+        for (int kf = 0; kf < NKF; ++kf) {
+            const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(&k_lds[krow0 * KP + kf * 32 + b * 8]);
+            const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(&k_lds[(krow0 + 4) * KP + kf * 32 + b * 8]);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[kf], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qf[kf], s1, 0, 0, 0);
+        }
+        float sc[8];
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int kp = t0 + 8 * b + e;
+            const float raw = e < 4 ? s0[e] : s1[e - 4];
+            const bool seen = col_ok && kp >= qlo && kp <= qpos;
+            sc[e] = seen ? raw * scale2 : -INFINITY;
+            tile_max = fmaxf(tile_max, sc[e]);
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLR_WAVE));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLR_WAVE));
+        const float new_max = fmaxf(run_max, tile_max);
+        const float corr = new_max > -INFINITY ? exp2f(run_max - new_max) : 1.f;
+        float part = 0.f;
+        bf16x8 pf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float p = new_max > -INFINITY ? exp2f(sc[e] - new_max) : 0.f;      // (exp2(-inf) = 0 for unseen keys)
+            part += p;
+            pf[e] = (__bf16)p;
+        }
+        part += __shfl_xor(part, 16, MLR_WAVE);
+        part += __shfl_xor(part, 32, MLR_WAVE);
+        run_sum = run_sum * corr + part;
+        run_max = new_max;
+#pragma unroll
+        for (int j = 0; j < NACC; ++j) {
+            const int vt = SPLITV ? j * 4 + wave : j;
+            if (vt * 16 < V) {                     // (the same in every lane)
+                acc[j] *= corr;
+                const bf16x8 av = *reinterpret_cast<const bf16x8*>(&vt_lds[(vt * 16 + i16) * VT_PITCH + 8 * b]);
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pf, acc[j], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    // the sink, and the division
+    float top = run_max, den = run_sum, f = 1.f;
+    if (a.sink != nullptr) {
+        const float sk = a.sink[head] * 1.4426950408889634f;
+        top = fmaxf(run_max, sk);
+        f = run_max > -INFINITY ? exp2f(run_max - top) : 0.f;
+        den = run_sum * f + exp2f(sk - top);
+    }
+    f = den > 0.f ? f / den : 0.f;
+    if (!col_ok) return;
+    __bf16* dst = a.out + (size_t)m * a.out_stride + (size_t)head * V;
+#pragma unroll
+    for (int j = 0; j < NACC; ++j) {
+        const int vt = SPLITV ? j * 4 + wave : j;
+        if (vt * 16 < V) {
+            // accumulator element r of a lane: channel vt * 16 + 4 b + r of column lane % 16
+            alignas(8) __bf16 four[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) four[r] = (__bf16)(acc[j][r] * f);
+            *reinterpret_cast<uint2*>(dst + vt * 16 + 4 * b) = *reinterpret_cast<const uint2*>(four);
+        }
+    }
+}
+
+template <int NKF, int NVT, bool SPLITV>
+static int launch_sink_tiles(const SinkArgs& a, const int32_t* first, const int32_t* count, int groups, int head_block,
+                             int head_blocks, hipStream_t stream) {
+    const size_t lds = ((size_t)TK * (NKF * 32 + 8) + (size_t)NVT * 16 * VT_PITCH) * sizeof(__bf16);
+    static bool raised = false;
+    if (!raised && lds > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&sink_attention_tiles_kernel<NKF, NVT, SPLITV>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+            return -3;
+        raised = true;
+    }
+    sink_attention_tiles_kernel<NKF, NVT, SPLITV><<<dim3(groups, a.kv_heads * head_blocks), 256, lds, stream>>>(
+        a, first, count, head_block, head_blocks);
+    return (int)hipGetLastError();
+}
+#endif
+
 extern "C" {
 
 int mlr_sink_attention(const void* q, long q_stride, const void* k_pages, long k_row, const void* v_pages, long v_row,
@@ -280,6 +494,47 @@ int mlr_latent_prep(const void* proj, long ld, void* q_out, void* pages, long ro
         (const elem_t*)proj, ld, (elem_t*)q_out, (elem_t*)pages, row_width, block_table, max_blocks, slots, positions,
         norm_w, eps, rope, heads, dim, rot, rank, page_size, write_cache);
     return (int)hipGetLastError();
+}
+
+// The matrix-core kernel over `groups` groups of consecutive tokens of one request each (group_first / group_count:
+// device vectors), every group holding at most 64 / head_block tokens (16 / head_block with split_values, which
+// deals the value channels out to the four wavefronts: single tokens).  head_block: a power of two, query heads of
+// one kv head side by side in a workgroup's columns.  Returns 1 when the sizes are not this kernel's.
+int mlr_sink_attention_tiles(const void* q, long q_stride, const void* k_pages, long k_row, const void* v_pages,
+                             long v_row, const int32_t* block_table, int max_blocks, const int32_t* slots,
+                             const int32_t* positions, const float* sink, void* out, long out_stride,
+                             const int32_t* group_first, const int32_t* group_count, int groups, int head_block,
+                             int split_values, int q_heads, int kv_heads, int key_dim, int value_dim, int page_size,
+                             int mask_kind, int mask_size, float scale, hipStream_t stream) {
+#if MLR_BF16
+    if (groups <= 0) return 0;
+    if (key_dim % 8 != 0 || value_dim % 16 != 0 || key_dim > 576 || value_dim > 512 || k_row % 8 != 0 || v_row % 8 != 0 ||
+        q_stride % 8 != 0 || out_stride % 4 != 0 || kv_heads <= 0 || q_heads % kv_heads != 0)
+        return 1;
+    if (head_block < 1 || head_block > (split_values ? 16 : 64) || (head_block & (head_block - 1)) != 0 ||
+        (mask_kind != MASK_ALL && mask_size <= 0))
+        return -1;
+    const int hg = q_heads / kv_heads, head_blocks = (hg + head_block - 1) / head_block;
+    if ((long)kv_heads * head_blocks > 65535) return -2;
+    SinkArgs a{(const elem_t*)q, q_stride, (const elem_t*)k_pages, k_row, (const elem_t*)v_pages, v_row, block_table,
+               slots, positions, sink, (elem_t*)out, out_stride, max_blocks, q_heads, kv_heads, key_dim, value_dim,
+               page_size, mask_kind, mask_size, scale};
+    const int nkf = (key_dim + 31) / 32, nvt = value_dim / 16;
+#define MLR_SINK_CLASS(NKF, NVT)                                                                                       \
+    if (nkf <= NKF && nvt <= NVT)                                                                                      \
+        return split_values ? launch_sink_tiles<NKF, NVT, true>(a, group_first, group_count, groups, head_block,      \
+                                                                 head_blocks, stream)                                  \
+                            : launch_sink_tiles<NKF, NVT, false>(a, group_first, group_count, groups, head_block,     \
+                                                                  head_blocks, stream);
+    MLR_SINK_CLASS(2, 4)
+    MLR_SINK_CLASS(4, 8)
+    MLR_SINK_CLASS(8, 16)
+    MLR_SINK_CLASS(18, 32)
+#undef MLR_SINK_CLASS
+    return 1;
+#else
+    return 1;
+#endif
 }
 
 }  // extern "C"

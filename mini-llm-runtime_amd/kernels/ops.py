@@ -1130,6 +1130,57 @@ class Kernels:
             _c_int(value_dim), _c_int(page_size), _c_int(kind), _c_int(int(mask_size)), _c_float(scale), _stream()),
             "sink_attention")
 
+    def sink_tiles_supported(self, key_dim, value_dim, k_row, v_row):
+        """Whether the matrix-core kernel takes these sizes: the bfloat16 engine, keys in multiples of 8 channels up to
+        576, values in multiples of 16 up to 512, cache rows that start at multiples of 16 bytes."""
+        return (self.dtype == torch.bfloat16 and key_dim % 8 == 0 and value_dim % 16 == 0 and key_dim <= 576
+                and value_dim <= 512 and k_row % 8 == 0 and v_row % 8 == 0)
+
+    @staticmethod
+    def sink_tiles_layout(q_heads, kv_heads):
+        """(heads side by side, tokens a group) of the matrix-core kernel's workgroups, for prompt portions (64 columns)
+        and for single tokens and short portions (16 columns, `split_values`)."""
+        per = q_heads // kv_heads
+        p2 = 1
+        while p2 < per:
+            p2 *= 2
+        big, small = min(p2, 64), min(p2, 16)
+        return big, 64 // big, small, 16 // small
+
+    @timed("attention")
+    def sink_attention_tiles(self, q, k_pages, v_pages, block_table, slots, positions, sink, out, group_first, group_count,
+                             groups, head_block, split_values, q_heads, kv_heads, key_dim, value_dim, page_size, scale,
+                             mask=None, mask_size=0):
+        """`sink_attention` on the matrix cores for `groups` groups of consecutive tokens of one request each (device
+        vectors group_first, group_count), at most 64 / head_block tokens a group (16 / head_block with
+        `split_values`)."""
+        _tensor(q, "q", self.dtype, ndim=2)
+        rows = q.shape[0]
+        _need(q.shape[1] == q_heads * key_dim, "q: wrong width")
+        k_row = self._sink_pages(k_pages, "k_pages", kv_heads, page_size, key_dim)
+        v_row = self._sink_pages(v_pages, "v_pages", kv_heads, page_size, value_dim)
+        _need(self.sink_tiles_supported(key_dim, value_dim, k_row, v_row) and q.shape[1] % 8 == 0,
+              "sink_attention_tiles: sizes that the matrix-core kernel does not take")
+        _need(mask in self.SINK_MASKS, f"mask {mask!r}: one of all, window, chunk")
+        kind = self.SINK_MASKS[mask]
+        _need(kind == 0 or mask_size >= 1, "a window or chunk needs a positive size")
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _tensor(positions, "positions", torch.int32, (rows,))
+        _tensor(group_first, "group_first", torch.int32, ndim=1)
+        _tensor(group_count, "group_count", torch.int32, ndim=1)
+        _need(group_first.numel() >= groups and group_count.numel() >= groups, "group vectors too short")
+        if sink is not None:
+            _tensor(sink, "sink", torch.float32, (q_heads,))
+        _tensor(out, "out", self.dtype, (rows, q_heads * value_dim))
+        code = self._lib("sink_attention").mlr_sink_attention_tiles(
+            _p(q), ctypes.c_long(q.shape[1]), _p(k_pages), ctypes.c_long(k_row), _p(v_pages), ctypes.c_long(v_row),
+            _p(block_table), _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(sink), _p(out),
+            ctypes.c_long(out.shape[1]), _p(group_first), _p(group_count), _c_int(groups), _c_int(head_block),
+            _c_int(1 if split_values else 0), _c_int(q_heads), _c_int(kv_heads), _c_int(key_dim), _c_int(value_dim),
+            _c_int(page_size), _c_int(kind), _c_int(int(mask_size)), _c_float(scale), _stream())
+        _ok(code, "sink_attention_tiles")
+
     # -- many small products, routing ----------------------------------------------------------
     GROUPED_ACTS = {None: 0, "relu_squared": 1}
     MAX_EXPERTS = 256

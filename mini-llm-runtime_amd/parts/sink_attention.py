@@ -44,6 +44,32 @@ def _rope_table(position, ctx, device, rot_limit):
     return rotation.table
 
 
+def _groups_plan(rows, q_heads, kv_heads):
+    """The token-group vectors that `attend` asks the step's context for."""
+    from ..kernels.ops import Kernels
+    _, big_tokens, _, small_tokens = Kernels.sink_tiles_layout(q_heads, kv_heads)
+    return {(f"token_groups_{small_tokens}_{max(1, big_tokens // small_tokens)}", torch.int32): 2 * rows + 2}
+
+
+def attend(ctx, q, k_pages, v_pages, view, sink, out, q_heads, kv_heads, key_dim, value_dim, scale, mask, mask_size):
+    """Every token of the step over the keys it sees.  The bfloat16 engine on the matrix cores where they take the
+    sizes (prompt portions in workgroups of 64 columns, single tokens and short portions in workgroups of 16 whose
+    wavefronts share the value channels); else, and in the float engine, one wavefront a (token, head), whose sums
+    follow from the token's position alone."""
+    k = ctx.kernels
+    if k.sink_tiles_supported(key_dim, value_dim, k_pages.shape[3], v_pages.shape[3]) and q.shape[1] % 8 == 0:
+        big_heads, big_tokens, small_heads, small_tokens = k.sink_tiles_layout(q_heads, kv_heads)
+        small, big, _ = ctx.token_groups(small_tokens, max(1, big_tokens // small_tokens))
+        for (first, count, n), heads, split in ((big, big_heads, False), (small, small_heads, True)):
+            if n:
+                k.sink_attention_tiles(q, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, sink, out, first,
+                                       count, n, heads, split, q_heads, kv_heads, key_dim, value_dim, view.page_size,
+                                       scale, mask, mask_size)
+        return
+    k.sink_attention(q, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, sink, out, q_heads, kv_heads,
+                     key_dim, value_dim, view.page_size, scale, mask, mask_size)
+
+
 @register_part("mixer", "sink_attention")
 class SinkAttention:
     graph_safe = True
@@ -94,7 +120,8 @@ class SinkAttention:
     def workspace_plan(self, rows, dtype, limits):
         s = self.spec
         return {("sink_proj", dtype): rows * (self.q_width + self.k_width + self.v_width), ("q", dtype): rows * self.q_width,
-                ("attn", dtype): rows * self.o_width, ("mixer_out", dtype): rows * s.hidden}
+                ("attn", dtype): rows * self.o_width, ("mixer_out", dtype): rows * s.hidden,
+                **_groups_plan(rows, s.q_heads, s.kv_heads)}
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
@@ -110,8 +137,8 @@ class SinkAttention:
                         self.k_norm, s.qk_norm.eps if s.qk_norm is not None else 0.0, rope, s.q_heads, s.kv_heads,
                         s.head_dim, s.value_dim, view.page_size, write_cache)
         attn = ctx.workspace.get("attn", (m, self.o_width), x.dtype)
-        k.sink_attention(q, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, self.sink, attn, s.q_heads,
-                         s.kv_heads, s.head_dim, s.value_dim, view.page_size, float(s.scale), self.mask, self.mask_size)
+        attend(ctx, q, k_pages, v_pages, view, self.sink, attn, s.q_heads, s.kv_heads, s.head_dim, s.value_dim,
+               float(s.scale), self.mask, self.mask_size)
         out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
         k.gemm(attn, self.o, out)
         return out
@@ -162,7 +189,7 @@ class LatentAttention:
         s = self.spec
         return {("latent_proj", dtype): rows * (self.q_width + self.row), ("latent_q", dtype): rows * s.heads * self.row,
                 ("latent_out", dtype): rows * s.heads * s.rank, ("attn", dtype): rows * self.o_width,
-                ("mixer_out", dtype): rows * s.hidden}
+                ("mixer_out", dtype): rows * s.hidden, **_groups_plan(rows, s.heads, 1)}
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
@@ -181,8 +208,8 @@ class LatentAttention:
         k.heads_gemm(torch.as_strided(proj, (m, s.heads, s.head_dim), (ld, s.head_dim + s.rot_dim, 1)), self.uk_t,
                      torch.as_strided(q, (m, s.heads, s.rank), (s.heads * self.row, self.row, 1)))
         lat = ctx.workspace.get("latent_out", (m, s.heads * s.rank), x.dtype)
-        k.sink_attention(q, pages, pages, view.block_table, ctx.slots, ctx.positions, self.sink, lat, s.heads, 1, self.row,
-                         s.rank, view.page_size, float(s.scale), self.mask, self.mask_size)
+        attend(ctx, q, pages, pages, view, self.sink, lat, s.heads, 1, self.row, s.rank, float(s.scale), self.mask,
+               self.mask_size)
         attn = ctx.workspace.get("attn", (m, self.o_width), x.dtype)
         k.heads_gemm(lat.view(m, s.heads, s.rank), self.uv, attn.view(m, s.heads, s.value_dim))
         out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)

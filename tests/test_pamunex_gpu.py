@@ -211,6 +211,47 @@ def test_sink_attention_finds_one_key_wherever_it_lies(dtype_name, kind, size, h
     assert 0 < seen_pairs and (kind == "all" or seen_pairs < len(pairs))       # both sides of the edge were asked
 
 
+def groups_of(count_rows, size):
+    first = list(range(0, count_rows, size))
+    count = [min(size, count_rows - f) for f in first]
+    return (torch.tensor(first, dtype=torch.int32, device="cuda"), torch.tensor(count, dtype=torch.int32, device="cuda"), len(first))
+
+
+@pytest.mark.parametrize("kind,size", [("window", 37), ("chunk", 24), ("window", 1), ("chunk", 1), ("all", 0), ("window", 150), ("chunk", 64)])
+@pytest.mark.parametrize("heads,kv,dim,vdim,shared,page", [(4, 2, 32, 16, False, 8), (3, 1, 24, 80, False, 4), (8, 8, 64, 64, False, 16),
+                                                           (5, 1, 112, 96, True, 16), (16, 1, 200, 160, True, 8), (2, 1, 576, 512, True, 16),
+                                                           (96, 1, 40, 32, True, 8)])
+def test_matrix_core_attention_in_groups_of_tokens_and_of_single_tokens(kind, size, heads, kv, dim, vdim, shared, page):
+    """Every position of a request of 210 tokens at once, in the workgroups of prompt portions (groups of consecutive
+    tokens) and in those of single tokens (groups of one token, and of a few), against the plain softmax; the value rows
+    of their own or inside the key rows."""
+    from mini_llm_runtime_amd.kernels import Kernels
+    dtype = torch.bfloat16
+    k = Kernels(dtype)
+    rng = np.random.default_rng(12)
+    T = 210
+    rows = as_rounded(rng.normal(size=(T, kv, dim)) * 0.5, dtype)
+    values = rows[:, :, :vdim] if shared else as_rounded(rng.normal(size=(T, kv, vdim)), dtype)
+    q = as_rounded(rng.normal(size=(T, heads, dim)) * 0.5, dtype)
+    sink = rng.normal(size=heads)
+    k_pages, table = paged(rows, page, dtype, seed=3)
+    v_pages = k_pages if shared else paged(values, page, dtype, seed=3)[0]
+    want = plain_attend(q, rows, values, np.arange(T), kind, size, sink, 0.25, heads // kv)
+    zeros, positions = torch.zeros(T, dtype=torch.int32, device="cuda"), torch.arange(T, dtype=torch.int32, device="cuda")
+    big_heads, big_tokens, small_heads, small_tokens = k.sink_tiles_layout(heads, kv)
+    assert k.sink_tiles_supported(dim, vdim, k_pages.shape[3], v_pages.shape[3])
+    for head_block, tokens, split in ((big_heads, big_tokens, False), (small_heads, small_tokens, True), (small_heads, 1, True),
+                                      (big_heads, 1, False)):
+        out = torch.full((T, heads * vdim), float("nan"), dtype=dtype, device="cuda")
+        first, count, n = groups_of(T, tokens)
+        k.sink_attention_tiles(on_gpu(q.reshape(T, -1), dtype), k_pages, v_pages, table, zeros, positions,
+                               on_gpu(sink, torch.float32), out, first, count, n, head_block, split, heads, kv, dim, vdim, page,
+                               0.25, None if kind == "all" else kind, size)
+        got = out.double().cpu().numpy()
+        assert np.isfinite(got).all(), (head_block, tokens, split)
+        np.testing.assert_allclose(got, want, rtol=3e-2, atol=2e-2, err_msg=str((head_block, tokens, split)))
+
+
 @pytest.mark.parametrize("dtype_name", DTYPES)
 def test_sink_attention_without_a_sink_and_with_values_inside_the_key_rows(dtype_name):
     """sink None is the usual softmax; values may be the first channels of the key rows themselves."""
