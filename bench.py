@@ -22,6 +22,8 @@ many gigabytes).  Every runner is built with the product's own defaults.  One JS
   * --only taletar: a line of its own: prefill and decode of Taletar models (Mamba-2, differential attention and
     gated linear attention layers) at two layer sizes beside a Qwen3 dense model of the same width, heads,
     feed-forward and layers, with milliseconds per kernel class.  The default workload is not touched by it.
+  * --only pamunex: the same for Pamunex models (latent attention over a sliding window beside a dense feed-forward,
+    chunked grouped-query attention beside a mixture of experts, in turn).
 """
 import argparse
 import json
@@ -480,20 +482,98 @@ class TaletarBench(Bench):
                     frac=round(step_bytes / (seconds / steps) / HBM_PEAK, 5)), step_bytes, report
 
 
+# `--only pamunex`: layer sizes that resemble a real model's, for a Pamunex model whose layers take latent attention
+# over a sliding window beside a dense feed-forward and chunked grouped-query attention beside a mixture of experts in
+# turn (norms behind the sublayers, a sink in every softmax), and for the closest model the engine had before, a
+# Qwen3 dense decoder of the same width, heads and number of layers.  The dense feed-forward has two matrices where
+# Qwen3's has three, so its inner size is one and a half times Qwen3's: equal weights a layer; an expert is a quarter
+# of that and a token uses two of eight.
+PAMUNEX_SIZES = {
+    "2k": dict(width=2048, ff=5632, vocab=32000, layers=8, heads=16, kv_heads=4, rank=512, window=1024, chunk=1024),
+    "4k": dict(width=4096, ff=12288, vocab=32000, layers=8, heads=32, kv_heads=8, rank=512, window=1024, chunk=1024),
+}
+
+
+class PamunexBench(Bench):
+    """A Pamunex model of PAMUNEX_SIZES[size] with random weights drawn on the GPU."""
+
+    def __init__(self, size, args):
+        import torch
+        from mini_llm_runtime_amd.api import parse_dtype
+        from mini_llm_runtime_amd.config import config_from_dict
+        from mini_llm_runtime_amd.parts import DecoderModel, expected_tensors
+        from mini_llm_runtime_amd.weights import random_tensors_on_device
+        d = PAMUNEX_SIZES[size]
+        self.torch, self.args, self.size = torch, args, size
+        self.dtype = parse_dtype(args.dtype)
+        self.tag = "bf16" if self.dtype == torch.bfloat16 else "fp32"
+        latent = dict(type="latent_attention",
+                      mixer=dict(heads=d["heads"], dim=128, rot_dim=64, vdim=128, kv_rank=d["rank"], scale=192 ** -0.5,
+                                 rot=dict(dims=64, base=10000.0), mask=dict(size=d["window"])),
+                      mlp=dict(kind="dense", ff=d["ff"] * 3 // 2))
+        chunked = dict(type="attention",
+                       mixer=dict(heads=d["heads"], kv_heads=d["kv_heads"], dim=128, vdim=128, scale=128 ** -0.5,
+                                  rot=dict(dims=64, base=1000000.0), mask=dict(size=d["chunk"])),
+                       mlp=dict(kind="moe", expert=dict(ff=d["ff"] * 3 // 8),
+                                router=dict(experts=8, top=2, groups=dict(count=4, keep=2))))
+        self.layers = self.full_layers = d["layers"]
+        layers = [latent if i % 2 == 0 else chunked for i in range(self.layers)]
+        self.cfg = config_from_dict(dict(architecture="Pamunex", vocab=d["vocab"], width=d["width"], norm=dict(eps=1e-5),
+                                         logit_scale=0.5, layers=layers))
+        self.model = DecoderModel(self.cfg, random_tensors_on_device(expected_tensors(self.cfg), 0, self.dtype, "cuda"),
+                                  self.dtype, "cuda:0")
+        self.weights_from = "drawn on the GPU"
+        self.elem = 2 if self.dtype == torch.bfloat16 else 4
+        n_latent = (self.layers + 1) // 2
+        n_chunked = self.layers // 2
+        w, ff = d["width"], d["ff"]
+        # weights that a decoding step reads: everything but six of a routed layer's eight experts (at most: the
+        # tokens of a batch choose their own), the table once (as the head)
+        expert = 2 * w * (ff * 3 // 8)
+        self.weight_bytes = self.model.weight_bytes() - n_chunked * 6 * expert * self.elem
+        # cache rows that a decoding token's attention reads: the latent row once for all heads, keys and values of the
+        # kv heads; at most the window / the chunk's share of the context
+        self.latent_row_bytes = n_latent * (d["rank"] + 64) * self.elem
+        self.kv_row_bytes = n_chunked * d["kv_heads"] * 2 * 128 * self.elem
+        self.kv_bytes_per_token = 0                  # (see decode_point)
+        self.matrix_params = (self.model.weight_bytes() // self.elem) - d["vocab"] * w - n_chunked * 6 * expert
+        h = d["heads"]
+        seen = lambda t, size: sum(min(p % size if size == d["chunk"] else size - 1, p) + 1 for p in range(t))
+        self.attention_flops = lambda t: (n_latent * 2.0 * seen(t, d["window"] + 0) * h * (2 * d["rank"] + 64)
+                                          + n_chunked * 2.0 * sum(p % d["chunk"] + 1 for p in range(t)) * h * 256)
+        self.vocab = d["vocab"]
+        self.g = torch.Generator().manual_seed(0)
+
+    def prefill_flops(self, t):
+        d = PAMUNEX_SIZES[self.size]
+        return 2.0 * t * self.matrix_params + self.attention_flops(t) + 2.0 * d["vocab"] * d["width"]
+
+    def decode_point(self, batch, steps, warmup, context=None):
+        d = PAMUNEX_SIZES[self.size]
+        seconds, mean_context, report = self.decode(batch, steps, warmup, context)
+        keys_latent = min(mean_context, d["window"])
+        keys_chunk = (mean_context % d["chunk"]) + 1
+        step_bytes = self.weight_bytes + batch * (keys_latent * self.latent_row_bytes + keys_chunk * self.kv_row_bytes)
+        return dict(tok_s=round(batch * steps / seconds, 1), ms=round(seconds / steps * 1e3, 4),
+                    frac=round(step_bytes / (seconds / steps) / HBM_PEAK, 5)), step_bytes, report
+
+
 def design_block(args):
     """Prefill (2048 tokens in one step) and decode (batch 8 and 64 behind --context tokens) of the Taletar sizes
     beside a Qwen3 dense model of equal width, heads, feed-forward and layers; then the same steps once more with
     events around every launch: milliseconds per kernel class."""
     import copy
     out = {}
-    for size in (args.design_sizes.split(",") if args.design_sizes else list(DESIGN_SIZES)):
-        d = DESIGN_SIZES[size]
+    design = getattr(args, "design", "taletar")
+    table, make_design = (PAMUNEX_SIZES, PamunexBench) if design == "pamunex" else (DESIGN_SIZES, TaletarBench)
+    for size in (args.design_sizes.split(",") if args.design_sizes else list(table)):
+        d = table[size]
         dense = (d["layers"], dict(hidden_size=d["width"], num_attention_heads=d["heads"], num_key_value_heads=d["kv_heads"],
                                    head_dim=128, intermediate_size=d["ff"], vocab_size=d["vocab"],
                                    max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1000000.0,
                                    tie_word_embeddings=False))
         block = {}
-        for name, make in (("taletar", lambda a: TaletarBench(size, a)), ("qwen3_dense", lambda a: Bench(size, 0, a, sizes=dense))):
+        for name, make in ((design, lambda a: make_design(size, a)), ("qwen3_dense", lambda a: Bench(size, 0, a, sizes=dense))):
             plain_args, profiled = copy.copy(args), copy.copy(args)
             plain_args.profile, plain_args.weights = False, "gpu"
             profiled.profile, profiled.weights, profiled.prefill_reps = True, "gpu", 3
@@ -534,12 +614,12 @@ def main():
                          "tensors drawn on the GPU; auto: folder for the 0.6B sizes, gpu for the larger ones")
     ap.add_argument("--warm-up", type=int, default=0,
                     help="--only engine: 1 captures the decoding steps (Engine.warm_up) before the first burst")
-    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prompt", "engine", "mixed", "taletar"],
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prompt", "engine", "mixed", "taletar", "pamunex"],
                     help="profiling aid: run just the decode steps, just the prefill or just the mixed step; prompt: one "
                          "prompt of --context tokens in portions of 2048; engine: the "
                          "scheduler over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "
                          "batch slots), printed as one line of its own")
-    ap.add_argument("--design-sizes", default="", help="--only taletar: which of its sizes (2k, 4k; default both)")
+    ap.add_argument("--design-sizes", default="", help="--only taletar / pamunex: which of its sizes (2k, 4k; default both)")
     ap.add_argument("--library", type=int, default=1,
                     help="0: every matrix product on the hand-written kernels, none in the vendor library")
     ap.add_argument("--split-keys", type=int, default=256, help="the smallest range of keys of one attention workgroup")
@@ -563,8 +643,9 @@ def main():
     if not args.tune:
         from mini_llm_runtime_amd.kernels import build
         build.load("library_gemm").mlr_library_gemm_tuning(0)
-    if args.only == "taletar":
-        print(json.dumps({"taletar_sizes": design_block(args), "context": args.context, "dtype": args.dtype}))
+    if args.only in ("taletar", "pamunex"):
+        args.design = args.only
+        print(json.dumps({f"{args.only}_sizes": design_block(args), "context": args.context, "dtype": args.dtype}))
         return 0
     bench = Bench(args.size, args.layers, args)
     c = bench.cfg

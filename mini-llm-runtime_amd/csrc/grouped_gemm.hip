@@ -231,11 +231,22 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const elem_t* __restric
     __shared__ float g_lds[MAX_EXPERTS];
     const int m = blockIdx.x, lane = threadIdx.x;
     const elem_t* row = x + (size_t)m * ldx;
-    for (int e = 0; e < experts; ++e) {
-        float part = 0.f;
-        for (int i = lane; i < width; i += 64) part = fmaf(to_float(row[i]), router[(size_t)e * width + i], part);
-        part = wave_sum(part);
-        if (lane == 0) s_lds[e] = 1.0f / (1.0f + expf(-part));
+    // eight experts a pass over the row: a lane's sum for an expert takes the row's elements in ascending order
+    for (int e0 = 0; e0 < experts; e0 += 8) {
+        float part[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) part[j] = 0.f;
+        for (int i = lane; i < width; i += 64) {
+            const float xv = to_float(row[i]);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (e0 + j < experts) part[j] = fmaf(xv, router[(size_t)(e0 + j) * width + i], part[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float z = wave_sum(part[j]);
+            if (lane == 0 && e0 + j < experts) s_lds[e0 + j] = 1.0f / (1.0f + expf(-z));
+        }
     }
     __syncthreads();
     const int per = experts / group_count;

@@ -40,6 +40,10 @@ struct SinkArgs {
     elem_t* out; long out_stride;              // out[m * out_stride + head * value_dim + c]
     int max_blocks, q_heads, kv_heads, key_dim, value_dim, page_size, mask_kind, mask_size;
     float scale;
+    // key ranges over several workgroups (the matrix-core kernel): workgroup z of a group takes split_keys keys from
+    // the group's first tile on and leaves (unnormalised values, maximum, sum) in partial[((g * tokens + i) * q_heads +
+    // head) * splits + z][value_dim + 4] for token i of group g; null: one workgroup walks every key and writes out
+    float* partial; int split_keys, splits, group_tokens;
 };
 
 __device__ __forceinline__ int first_seen(int pos, int kind, int size) {
@@ -249,7 +253,10 @@ __global__ __launch_bounds__(64) void latent_prep_kernel(
 // from the first key of the group's first token to the last token's own position, in tiles of 32 keys at absolute
 // multiples of 32; a tile's key rows are staged once through LDS for all its columns (row-major for the scores,
 // and the value channels transposed, [channel][key], for the second product: 16-byte reads of eight keys of one
-// channel), the next tile's rows on their way from memory into registers meanwhile.  Where the value rows ARE the
+// channel), the next tile's rows on their way from memory into registers meanwhile.  A thread stages 16 bytes (eight
+// channels of one key); consecutive lanes take consecutive KEYS, so that the eight 2-byte writes that transpose
+// them land in different LDS banks (lanes that take consecutive channels of one key all meet in two banks, which
+// made a tile's staging ten times as long as its products).  Where the value rows ARE the
 // key rows they are read once.  Rows outside the range, or without a page, are staged as zeros.
 //   S^T = K Q^T with v_mfma_f32_16x16x32_bf16: row i of the instruction's first operand is tile key
 //   8 (i / 4) + 4 s + i % 4 of half-tile s, so that a lane ends up with the scores of the eight CONSECUTIVE keys
@@ -262,6 +269,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 #define TK 32                   // keys in a tile
 #define VT_PITCH 40             // elements between the channels of the transposed values (80 bytes)
+#define TILES_MAX_BLOCKS 2048   // page ids of a workgroup's key range that it keeps in LDS
 
 template <int NKF, int NVT, bool SPLITV>
 __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, const int32_t* __restrict__ group_first,
@@ -274,6 +282,7 @@ __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, c
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     __bf16* k_lds = reinterpret_cast<__bf16*>(lds_raw);               // [TK][KP]
     __bf16* vt_lds = k_lds + TK * KP;                                  // [NVT * 16][VT_PITCH]
+    int32_t* page_lds = reinterpret_cast<int32_t*>(vt_lds + NVT * 16 * VT_PITCH);      // [TILES_MAX_BLOCKS]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int group = blockIdx.x, kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
     const int first = group_first[group], count = group_count[group];
@@ -281,7 +290,12 @@ __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, c
     const int D = a.key_dim, V = a.value_dim;
     const bool shared_rows = a.v_pages == a.k_pages;
     const int p0 = a.positions[first], slot = a.slots[first];
-    const int kbegin = first_seen(p0, a.mask_kind, a.mask_size), kend = p0 + count;
+    int kbegin = first_seen(p0, a.mask_kind, a.mask_size), kend = p0 + count;
+    if (a.partial != nullptr) {                // this workgroup's share of the keys, from the group's first tile on
+        const int base = (kbegin / TK) * TK + (int)blockIdx.z * a.split_keys;
+        kbegin = max(kbegin, base);
+        kend = min(kend, base + a.split_keys);
+    }
     const int32_t* table = a.block_table + (size_t)slot * a.max_blocks;
 
     // this lane's column
@@ -305,54 +319,60 @@ __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, c
     float run_max = -INFINITY, run_sum = 0.f;
     const float scale2 = a.scale * 1.4426950408889634f;
 
+    // the page ids of the workgroup's key range, once
+    const int block0 = kbegin / a.page_size;
+    const int n_blocks = kend > kbegin ? min((kend - 1) / a.page_size - block0 + 1, TILES_MAX_BLOCKS) : 0;
+    for (int i = tid; i < n_blocks; i += 256) page_lds[i] = block0 + i < a.max_blocks ? table[block0 + i] : -1;
+    __syncthreads();
+
+    // A thread stages the same key of every tile (key = thread % 32: 256 is a multiple of it) and the chunks
+    // thread / 32 + 8 i of its row: one row address a tile, then loads that do not wait for each other (addresses
+    // are clamped and what must not count is zeroed afterwards: a load behind a branch would wait for the one before).
     bf16x8 kreg[NSK], vreg[NSV];
-    auto row_of_key = [&](int kp) -> long long {
-        if (kp < kbegin || kp >= kend) return -1;
-        const int block = kp / a.page_size;
-        const int page = block < a.max_blocks ? table[block] : -1;
-        return page < 0 ? -1 : ((long long)page * a.kv_heads + kvh) * a.page_size + kp % a.page_size;
-    };
+    const int my_key = tid & 31, my_chunk = tid >> 5;
     auto fetch = [&](int t0) {
+        const int kp = t0 + my_key;
+        const bool inside = kp >= kbegin && kp < kend;
+        const int blk = inside ? kp / a.page_size - block0 : 0;
+        const int page = (inside && blk < n_blocks) ? page_lds[blk] : -1;
+        const bool have = page >= 0;
+        const long long r = have ? ((long long)page * a.kv_heads + kvh) * a.page_size + kp % a.page_size : 0;
+        const __bf16* krow = a.k_pages + r * a.k_row;
 #pragma unroll
         for (int i = 0; i < NSK; ++i) {
-            const int q = tid + 256 * i, key = q / CPK, d = (q % CPK) * 8;
-            kreg[i] = zero8;
-            if (q < TK * CPK && d < D) {
-                const long long r = row_of_key(t0 + key);
-                if (r >= 0) kreg[i] = *reinterpret_cast<const bf16x8*>(a.k_pages + r * a.k_row + d);
-            }
+            const int d = (my_chunk + 8 * i) * 8;
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(krow + min(d, D - 8));
+            kreg[i] = (have && d < D) ? v : zero8;
         }
         if (!shared_rows) {
+            const __bf16* vrow = a.v_pages + r * a.v_row;
 #pragma unroll
             for (int i = 0; i < NSV; ++i) {
-                const int q = tid + 256 * i, key = q / CPV, d = (q % CPV) * 8;
-                vreg[i] = zero8;
-                if (q < TK * CPV && d < V) {
-                    const long long r = row_of_key(t0 + key);
-                    if (r >= 0) vreg[i] = *reinterpret_cast<const bf16x8*>(a.v_pages + r * a.v_row + d);
-                }
+                const int d = (my_chunk + 8 * i) * 8;
+                const bf16x8 v = *reinterpret_cast<const bf16x8*>(vrow + min(d, V - 8));
+                vreg[i] = (have && d < V) ? v : zero8;
             }
         }
     };
     auto stage = [&]() {
 #pragma unroll
         for (int i = 0; i < NSK; ++i) {
-            const int q = tid + 256 * i, key = q / CPK, d = (q % CPK) * 8;
-            if (q < TK * CPK) {
-                *reinterpret_cast<bf16x8*>(&k_lds[key * KP + d]) = kreg[i];
+            const int d = (my_chunk + 8 * i) * 8;
+            if (d < KD) {
+                *reinterpret_cast<bf16x8*>(&k_lds[my_key * KP + d]) = kreg[i];
                 if (shared_rows && d < NVT * 16) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) vt_lds[(d + e) * VT_PITCH + key] = (d + e < V) ? kreg[i][e] : (__bf16)0.f;
+                    for (int e = 0; e < 8; ++e) vt_lds[(d + e) * VT_PITCH + my_key] = (d + e < V) ? kreg[i][e] : (__bf16)0.f;
                 }
             }
         }
         if (!shared_rows) {
 #pragma unroll
             for (int i = 0; i < NSV; ++i) {
-                const int q = tid + 256 * i, key = q / CPV, d = (q % CPV) * 8;
-                if (q < TK * CPV) {
+                const int d = (my_chunk + 8 * i) * 8;
+                if (d < NVT * 16) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) vt_lds[(d + e) * VT_PITCH + key] = vreg[i][e];
+                    for (int e = 0; e < 8; ++e) vt_lds[(d + e) * VT_PITCH + my_key] = vreg[i][e];
                 }
             }
         }
@@ -412,6 +432,20 @@ __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, c
         }
         __syncthreads();
     }
+    if (a.partial != nullptr) {                // this range's share: the merge kernel finishes the column
+        if (!col_ok) return;
+        float* dst = a.partial + ((((size_t)group * a.group_tokens + ti) * a.q_heads + head) * a.splits + blockIdx.z) * (V + 4);
+#pragma unroll
+        for (int j = 0; j < NACC; ++j) {
+            const int vt = SPLITV ? j * 4 + wave : j;
+            if (vt * 16 < V) *reinterpret_cast<float4*>(dst + vt * 16 + 4 * b) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+        }
+        if (b == 0 && (!SPLITV || wave == 0)) {
+            dst[V] = run_max;
+            dst[V + 1] = run_sum;
+        }
+        return;
+    }
     // the sink, and the division
     float top = run_max, den = run_sum, f = 1.f;
     if (a.sink != nullptr) {
@@ -436,10 +470,47 @@ __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, c
     }
 }
 
+// The merge of the key ranges' shares (maxima and sums in the base-2 domain, as the kernel above leaves them), the
+// sink and the division: one wavefront per (token of a group, head).
+__global__ __launch_bounds__(64) void sink_tiles_combine_kernel(SinkArgs a, const int32_t* __restrict__ group_first,
+                                                                const int32_t* __restrict__ group_count) {
+    const int group = blockIdx.x, ti = blockIdx.z, head = blockIdx.y, lane = threadIdx.x;
+    if (ti >= group_count[group]) return;
+    const int m = group_first[group] + ti, V = a.value_dim;
+    const float* base = a.partial + (((size_t)group * a.group_tokens + ti) * a.q_heads + head) * a.splits * (V + 4);
+    float top = a.sink != nullptr ? a.sink[head] * 1.4426950408889634f : -INFINITY;
+    const float sink2 = top;
+    for (int z = 0; z < a.splits; ++z) top = fmaxf(top, base[(size_t)z * (V + 4) + V]);
+    float den = a.sink != nullptr ? exp2f(sink2 - top) : 0.f;
+    float num[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) num[i] = 0.f;
+    for (int z = 0; z < a.splits; ++z) {
+        const float* p = base + (size_t)z * (V + 4);
+        const float zmax = p[V];
+        if (!(zmax > -INFINITY)) continue;     // (a range beyond the token's keys)
+        const float w = exp2f(zmax - top);
+        den += w * p[V + 1];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int c = lane + 64 * i;
+            if (c < V) num[i] += w * p[c];
+        }
+    }
+    const float inv = den > 0.f ? 1.0f / den : 0.f;
+    __bf16* dst = a.out + (size_t)m * a.out_stride + (size_t)head * V;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int c = lane + 64 * i;
+        if (c < V) dst[c] = (__bf16)(num[i] * inv);
+    }
+}
+
 template <int NKF, int NVT, bool SPLITV>
 static int launch_sink_tiles(const SinkArgs& a, const int32_t* first, const int32_t* count, int groups, int head_block,
                              int head_blocks, hipStream_t stream) {
-    const size_t lds = ((size_t)TK * (NKF * 32 + 8) + (size_t)NVT * 16 * VT_PITCH) * sizeof(__bf16);
+    const size_t lds = ((size_t)TK * (NKF * 32 + 8) + (size_t)NVT * 16 * VT_PITCH) * sizeof(__bf16) +
+                       TILES_MAX_BLOCKS * sizeof(int32_t);
     static bool raised = false;
     if (!raised && lds > 48 * 1024) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(&sink_attention_tiles_kernel<NKF, NVT, SPLITV>),
@@ -447,8 +518,10 @@ static int launch_sink_tiles(const SinkArgs& a, const int32_t* first, const int3
             return -3;
         raised = true;
     }
-    sink_attention_tiles_kernel<NKF, NVT, SPLITV><<<dim3(groups, a.kv_heads * head_blocks), 256, lds, stream>>>(
-        a, first, count, head_block, head_blocks);
+    sink_attention_tiles_kernel<NKF, NVT, SPLITV><<<dim3(groups, a.kv_heads * head_blocks, a.partial ? a.splits : 1), 256, lds,
+                                                   stream>>>(a, first, count, head_block, head_blocks);
+    if (a.partial != nullptr)
+        sink_tiles_combine_kernel<<<dim3(groups, a.q_heads, a.group_tokens), 64, 0, stream>>>(a, first, count);
     return (int)hipGetLastError();
 }
 #endif
@@ -465,7 +538,7 @@ int mlr_sink_attention(const void* q, long q_stride, const void* k_pages, long k
         return -1;
     SinkArgs a{(const elem_t*)q, q_stride, (const elem_t*)k_pages, k_row, (const elem_t*)v_pages, v_row, block_table,
                slots, positions, sink, (elem_t*)out, out_stride, max_blocks, q_heads, kv_heads, key_dim, value_dim,
-               page_size, mask_kind, mask_size, scale};
+               page_size, mask_kind, mask_size, scale, nullptr, 0, 1, 1};
     sink_attention_kernel<<<dim3(rows, q_heads), 64, 0, stream>>>(a);
     return (int)hipGetLastError();
 }
@@ -499,15 +572,25 @@ int mlr_latent_prep(const void* proj, long ld, void* q_out, void* pages, long ro
 // The matrix-core kernel over `groups` groups of consecutive tokens of one request each (group_first / group_count:
 // device vectors), every group holding at most 64 / head_block tokens (16 / head_block with split_values, which
 // deals the value channels out to the four wavefronts: single tokens).  head_block: a power of two, query heads of
-// one kv head side by side in a workgroup's columns.  Returns 1 when the sizes are not this kernel's.
+// one kv head side by side in a workgroup's columns.  max_context: the longest context of the step (what a
+// workgroup walks at most when no mask bounds it).  splits > 1: a group's keys in `splits` ranges of split_keys keys
+// (a multiple of 32) from its first tile on, one workgroup each, their shares in `partial` (floats: groups x tokens a
+// group x q_heads x splits x (value_dim + 4)) merged by a second launch.  Returns 1 when the sizes are not this
+// kernel's.
 int mlr_sink_attention_tiles(const void* q, long q_stride, const void* k_pages, long k_row, const void* v_pages,
                              long v_row, const int32_t* block_table, int max_blocks, const int32_t* slots,
                              const int32_t* positions, const float* sink, void* out, long out_stride,
                              const int32_t* group_first, const int32_t* group_count, int groups, int head_block,
                              int split_values, int q_heads, int kv_heads, int key_dim, int value_dim, int page_size,
-                             int mask_kind, int mask_size, float scale, hipStream_t stream) {
+                             int mask_kind, int mask_size, int max_context, float scale, float* partial, int split_keys,
+                             int splits, hipStream_t stream) {
 #if MLR_BF16
     if (groups <= 0) return 0;
+    {
+        // the keys that one workgroup may have to walk: its page ids must fit what it keeps of them
+        const long reach = mask_kind == MASK_ALL ? (long)max_context : (long)mask_size + 64;
+        if (reach / page_size + 2 > TILES_MAX_BLOCKS) return 1;
+    }
     if (key_dim % 8 != 0 || value_dim % 16 != 0 || key_dim > 576 || value_dim > 512 || k_row % 8 != 0 || v_row % 8 != 0 ||
         q_stride % 8 != 0 || out_stride % 4 != 0 || kv_heads <= 0 || q_heads % kv_heads != 0)
         return 1;
@@ -518,7 +601,10 @@ int mlr_sink_attention_tiles(const void* q, long q_stride, const void* k_pages, 
     if ((long)kv_heads * head_blocks > 65535) return -2;
     SinkArgs a{(const elem_t*)q, q_stride, (const elem_t*)k_pages, k_row, (const elem_t*)v_pages, v_row, block_table,
                slots, positions, sink, (elem_t*)out, out_stride, max_blocks, q_heads, kv_heads, key_dim, value_dim,
-               page_size, mask_kind, mask_size, scale};
+               page_size, mask_kind, mask_size, scale, splits > 1 ? partial : nullptr, split_keys, splits > 1 ? splits : 1,
+               (split_values ? 16 : 64) / head_block};
+    if (splits > 1 && (partial == nullptr || split_keys <= 0 || split_keys % TK != 0 || splits > 65535 || a.group_tokens > 65535))
+        return -1;
     const int nkf = (key_dim + 31) / 32, nvt = value_dim / 16;
 #define MLR_SINK_CLASS(NKF, NVT)                                                                                       \
     if (nkf <= NKF && nvt <= NVT)                                                                                      \

@@ -1130,11 +1130,17 @@ class Kernels:
             _c_int(value_dim), _c_int(page_size), _c_int(kind), _c_int(int(mask_size)), _c_float(scale), _stream()),
             "sink_attention")
 
-    def sink_tiles_supported(self, key_dim, value_dim, k_row, v_row):
+    SINK_TILES_BLOCKS = 2048
+
+    def sink_tiles_supported(self, key_dim, value_dim, k_row, v_row, page_size=16, mask=None, mask_size=0, max_context=0):
         """Whether the matrix-core kernel takes these sizes: the bfloat16 engine, keys in multiples of 8 channels up to
-        576, values in multiples of 16 up to 512, cache rows that start at multiples of 16 bytes."""
+        576, values in multiples of 16 up to 512, cache rows that start at multiples of 16 bytes, and a key range of
+        one workgroup (the window or chunk and its tokens; without a mask the step's longest context) whose page ids
+        fit what the kernel keeps of them."""
+        reach = max_context if self.SINK_MASKS.get(mask, 0) == 0 else mask_size + 64
         return (self.dtype == torch.bfloat16 and key_dim % 8 == 0 and value_dim % 16 == 0 and key_dim <= 576
-                and value_dim <= 512 and k_row % 8 == 0 and v_row % 8 == 0)
+                and value_dim <= 512 and k_row % 8 == 0 and v_row % 8 == 0
+                and reach // page_size + 2 <= self.SINK_TILES_BLOCKS)
 
     @staticmethod
     def sink_tiles_layout(q_heads, kv_heads):
@@ -1150,18 +1156,19 @@ class Kernels:
     @timed("attention")
     def sink_attention_tiles(self, q, k_pages, v_pages, block_table, slots, positions, sink, out, group_first, group_count,
                              groups, head_block, split_values, q_heads, kv_heads, key_dim, value_dim, page_size, scale,
-                             mask=None, mask_size=0):
+                             mask=None, mask_size=0, max_context=0, partial=None, split_keys=0, splits=1):
         """`sink_attention` on the matrix cores for `groups` groups of consecutive tokens of one request each (device
         vectors group_first, group_count), at most 64 / head_block tokens a group (16 / head_block with
-        `split_values`)."""
+        `split_values`).  splits > 1: a group's keys in that many ranges of `split_keys` keys (a multiple of 32), one
+        workgroup each, merged by a second launch through `partial` (float, `sink_partial_numel` elements)."""
         _tensor(q, "q", self.dtype, ndim=2)
         rows = q.shape[0]
         _need(q.shape[1] == q_heads * key_dim, "q: wrong width")
         k_row = self._sink_pages(k_pages, "k_pages", kv_heads, page_size, key_dim)
         v_row = self._sink_pages(v_pages, "v_pages", kv_heads, page_size, value_dim)
-        _need(self.sink_tiles_supported(key_dim, value_dim, k_row, v_row) and q.shape[1] % 8 == 0,
-              "sink_attention_tiles: sizes that the matrix-core kernel does not take")
         _need(mask in self.SINK_MASKS, f"mask {mask!r}: one of all, window, chunk")
+        _need(self.sink_tiles_supported(key_dim, value_dim, k_row, v_row, page_size, mask, mask_size, max_context)
+              and q.shape[1] % 8 == 0, "sink_attention_tiles: sizes that the matrix-core kernel does not take")
         kind = self.SINK_MASKS[mask]
         _need(kind == 0 or mask_size >= 1, "a window or chunk needs a positive size")
         _tensor(block_table, "block_table", torch.int32, ndim=2)
@@ -1173,13 +1180,25 @@ class Kernels:
         if sink is not None:
             _tensor(sink, "sink", torch.float32, (q_heads,))
         _tensor(out, "out", self.dtype, (rows, q_heads * value_dim))
+        if splits > 1:
+            _tensor(partial, "partial", torch.float32, ndim=1)
+            tokens = (16 if split_values else 64) // head_block
+            _need(split_keys > 0 and split_keys % 32 == 0 and
+                  partial.numel() >= self.sink_partial_numel(groups, tokens, q_heads, value_dim, splits),
+                  "sink_attention_tiles: key ranges in multiples of 32 keys, and room for their shares")
         code = self._lib("sink_attention").mlr_sink_attention_tiles(
             _p(q), ctypes.c_long(q.shape[1]), _p(k_pages), ctypes.c_long(k_row), _p(v_pages), ctypes.c_long(v_row),
             _p(block_table), _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(sink), _p(out),
             ctypes.c_long(out.shape[1]), _p(group_first), _p(group_count), _c_int(groups), _c_int(head_block),
             _c_int(1 if split_values else 0), _c_int(q_heads), _c_int(kv_heads), _c_int(key_dim), _c_int(value_dim),
-            _c_int(page_size), _c_int(kind), _c_int(int(mask_size)), _c_float(scale), _stream())
+            _c_int(page_size), _c_int(kind), _c_int(int(mask_size)), _c_int(int(max_context)), _c_float(scale),
+            _p(partial if splits > 1 else None), _c_int(int(split_keys)), _c_int(int(splits)), _stream())
         _ok(code, "sink_attention_tiles")
+
+    @staticmethod
+    def sink_partial_numel(groups, tokens, q_heads, value_dim, splits):
+        """Floats that the shares of `splits` key ranges take for `groups` groups of up to `tokens` tokens."""
+        return groups * tokens * q_heads * splits * (value_dim + 4)
 
     # -- many small products, routing ----------------------------------------------------------
     GROUPED_ACTS = {None: 0, "relu_squared": 1}

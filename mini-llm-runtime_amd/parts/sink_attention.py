@@ -44,11 +44,35 @@ def _rope_table(position, ctx, device, rot_limit):
     return rotation.table
 
 
-def _groups_plan(rows, q_heads, kv_heads):
-    """The token-group vectors that `attend` asks the step's context for."""
+PARTIAL_CAP = 8 << 20         # floats that the shares of the key ranges of one launch may take at most
+RANGE_KEYS = 128              # the narrowest key range of a workgroup
+MOST_RANGES = 16              # key ranges of a group at most
+
+
+def _groups_plan(rows, q_heads, kv_heads, value_dim):
+    """The token-group vectors and the room for key ranges' shares that `attend` asks the step's context for."""
     from ..kernels.ops import Kernels
     _, big_tokens, _, small_tokens = Kernels.sink_tiles_layout(q_heads, kv_heads)
-    return {(f"token_groups_{small_tokens}_{max(1, big_tokens // small_tokens)}", torch.int32): 2 * rows + 2}
+    return {(f"token_groups_{small_tokens}_{max(1, big_tokens // small_tokens)}", torch.int32): 2 * rows + 2,
+            ("sink_partial", torch.float32): min(PARTIAL_CAP, Kernels.sink_partial_numel(rows, small_tokens, q_heads, value_dim, MOST_RANGES))}
+
+
+def _key_ranges(ctx, groups, tokens, workgroups, q_heads, value_dim, mask, mask_size):
+    """(keys a range, ranges, room for their shares) for a launch over `groups` groups of single tokens or short portions
+    that has `workgroups` workgroups without ranges: where those do not fill the GPU, a group's keys (its window or
+    chunk; without a mask the step's longest context) are dealt out to several workgroups, as many as reach
+    `target_workgroups`, none narrower than RANGE_KEYS, and no more than their shares have room for."""
+    k = ctx.kernels
+    reach = (mask_size if mask == "chunk" else mask_size + tokens - 1) if mask is not None else ctx.max_context
+    reach = min(reach, ctx.max_context + 31) + 31             # (ranges start at the first tile, which may start earlier)
+    most = max(1, min(MOST_RANGES, -(-reach // RANGE_KEYS), -(-ctx.target_workgroups // max(1, workgroups))))
+    room = ctx.workspace.get("sink_partial", (min(PARTIAL_CAP, k.sink_partial_numel(groups, tokens, q_heads, value_dim, most)),),
+                             torch.float32)
+    most = min(most, room.numel() // k.sink_partial_numel(groups, tokens, q_heads, value_dim, 1))
+    if most <= 1:
+        return 0, 1, None
+    keys = -(-(-(-reach // most)) // 32) * 32
+    return keys, -(-reach // keys), room
 
 
 def attend(ctx, q, k_pages, v_pages, view, sink, out, q_heads, kv_heads, key_dim, value_dim, scale, mask, mask_size):
@@ -57,14 +81,20 @@ def attend(ctx, q, k_pages, v_pages, view, sink, out, q_heads, kv_heads, key_dim
     wavefronts share the value channels); else, and in the float engine, one wavefront a (token, head), whose sums
     follow from the token's position alone."""
     k = ctx.kernels
-    if k.sink_tiles_supported(key_dim, value_dim, k_pages.shape[3], v_pages.shape[3]) and q.shape[1] % 8 == 0:
+    if k.sink_tiles_supported(key_dim, value_dim, k_pages.shape[3], v_pages.shape[3], view.page_size, mask, mask_size,
+                              ctx.max_positions) and q.shape[1] % 8 == 0:
         big_heads, big_tokens, small_heads, small_tokens = k.sink_tiles_layout(q_heads, kv_heads)
         small, big, _ = ctx.token_groups(small_tokens, max(1, big_tokens // small_tokens))
         for (first, count, n), heads, split in ((big, big_heads, False), (small, small_heads, True)):
-            if n:
-                k.sink_attention_tiles(q, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, sink, out, first,
-                                       count, n, heads, split, q_heads, kv_heads, key_dim, value_dim, view.page_size,
-                                       scale, mask, mask_size)
+            if n == 0:
+                continue
+            keys, ranges, room = (0, 1, None)
+            if split:
+                per_group = kv_heads * -(-(q_heads // kv_heads) // heads)
+                keys, ranges, room = _key_ranges(ctx, n, small_tokens, n * per_group, q_heads, value_dim, mask, mask_size)
+            k.sink_attention_tiles(q, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, sink, out, first,
+                                   count, n, heads, split, q_heads, kv_heads, key_dim, value_dim, view.page_size,
+                                   scale, mask, mask_size, ctx.max_positions, partial=room, split_keys=keys, splits=ranges)
         return
     k.sink_attention(q, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, sink, out, q_heads, kv_heads,
                      key_dim, value_dim, view.page_size, scale, mask, mask_size)
@@ -121,7 +151,7 @@ class SinkAttention:
         s = self.spec
         return {("sink_proj", dtype): rows * (self.q_width + self.k_width + self.v_width), ("q", dtype): rows * self.q_width,
                 ("attn", dtype): rows * self.o_width, ("mixer_out", dtype): rows * s.hidden,
-                **_groups_plan(rows, s.q_heads, s.kv_heads)}
+                **_groups_plan(rows, s.q_heads, s.kv_heads, s.value_dim)}
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
@@ -189,7 +219,7 @@ class LatentAttention:
         s = self.spec
         return {("latent_proj", dtype): rows * (self.q_width + self.row), ("latent_q", dtype): rows * s.heads * self.row,
                 ("latent_out", dtype): rows * s.heads * s.rank, ("attn", dtype): rows * self.o_width,
-                ("mixer_out", dtype): rows * s.hidden, **_groups_plan(rows, s.heads, 1)}
+                ("mixer_out", dtype): rows * s.hidden, **_groups_plan(rows, s.heads, 1, s.rank)}
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec

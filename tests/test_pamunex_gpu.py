@@ -239,17 +239,24 @@ def test_matrix_core_attention_in_groups_of_tokens_and_of_single_tokens(kind, si
     want = plain_attend(q, rows, values, np.arange(T), kind, size, sink, 0.25, heads // kv)
     zeros, positions = torch.zeros(T, dtype=torch.int32, device="cuda"), torch.arange(T, dtype=torch.int32, device="cuda")
     big_heads, big_tokens, small_heads, small_tokens = k.sink_tiles_layout(heads, kv)
-    assert k.sink_tiles_supported(dim, vdim, k_pages.shape[3], v_pages.shape[3])
-    for head_block, tokens, split in ((big_heads, big_tokens, False), (small_heads, small_tokens, True), (small_heads, 1, True),
-                                      (big_heads, 1, False)):
+    assert k.sink_tiles_supported(dim, vdim, k_pages.shape[3], v_pages.shape[3], page, None if kind == "all" else kind, size, T)
+    for head_block, tokens, split, ranges in ((big_heads, big_tokens, False, 0), (small_heads, small_tokens, True, 0),
+                                              (small_heads, 1, True, 0), (big_heads, 1, False, 0), (small_heads, small_tokens, True, 32),
+                                              (small_heads, 1, True, 96)):
         out = torch.full((T, heads * vdim), float("nan"), dtype=dtype, device="cuda")
         first, count, n = groups_of(T, tokens)
+        more = {}
+        if ranges:                                     # a group's keys in ranges of that many, one workgroup each
+            splits = -(-(T + 31) // ranges)
+            room = (16 if split else 64) // head_block
+            more = dict(partial=torch.full((k.sink_partial_numel(n, room, heads, vdim, splits),), float("nan"), device="cuda"),
+                        split_keys=ranges, splits=splits)
         k.sink_attention_tiles(on_gpu(q.reshape(T, -1), dtype), k_pages, v_pages, table, zeros, positions,
                                on_gpu(sink, torch.float32), out, first, count, n, head_block, split, heads, kv, dim, vdim, page,
-                               0.25, None if kind == "all" else kind, size)
+                               0.25, None if kind == "all" else kind, size, T, **more)
         got = out.double().cpu().numpy()
-        assert np.isfinite(got).all(), (head_block, tokens, split)
-        np.testing.assert_allclose(got, want, rtol=3e-2, atol=2e-2, err_msg=str((head_block, tokens, split)))
+        assert np.isfinite(got).all(), (head_block, tokens, split, ranges)
+        np.testing.assert_allclose(got, want, rtol=3e-2, atol=2e-2, err_msg=str((head_block, tokens, split, ranges)))
 
 
 @pytest.mark.parametrize("dtype_name", DTYPES)
