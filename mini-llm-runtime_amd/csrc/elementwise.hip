@@ -558,6 +558,7 @@ __global__ __launch_bounds__(256) void gated_part_norm_vec_kernel(const float* _
 //     cast != null also cast[src] = T(acc[src]): the stream as the next sublayer's input;
 //   else out[r] = T(y).
 // One workgroup a row.
+#define LN_REGS 16
 __global__ __launch_bounds__(256) void layernorm_kernel(const elem_t* __restrict__ xe, const float* __restrict__ xf,
                                                         const float* __restrict__ weight, const float* __restrict__ bias,
                                                         const int32_t* __restrict__ rows, float* __restrict__ acc,
@@ -568,18 +569,37 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const elem_t* __restrict
     const size_t src = rows ? (size_t)rows[r] : (size_t)r;
     const elem_t* re = xe ? xe + src * width : nullptr;
     const float* rf = xf ? xf + src * width : nullptr;
+    // the row is read once and kept in registers where it fits (up to LN_REGS values a thread), else read again
+    const bool kept = width <= LN_REGS * (int)blockDim.x;
+    float x[LN_REGS];
     float sum = 0.f;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) sum += re ? to_float(re[i]) : rf[i];
+    if (kept) {
+#pragma unroll
+        for (int j = 0; j < LN_REGS; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            x[j] = i < width ? (re ? to_float(re[i]) : rf[i]) : 0.f;
+            sum += x[j];
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) sum += re ? to_float(re[i]) : rf[i];
+    }
     const float mean = block_sum(sum, scratch) / (float)width;
     float dev = 0.f;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        const float d = (re ? to_float(re[i]) : rf[i]) - mean;
-        dev += d * d;
+    if (kept) {
+#pragma unroll
+        for (int j = 0; j < LN_REGS; ++j) {
+            const float d = threadIdx.x + j * blockDim.x < width ? x[j] - mean : 0.f;
+            dev += d * d;
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) {
+            const float d = (re ? to_float(re[i]) : rf[i]) - mean;
+            dev += d * d;
+        }
     }
     const float inv = 1.0f / sqrtf(block_sum(dev, scratch) / (float)width + eps);
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        const float x = re ? to_float(re[i]) : rf[i];
-        const float y = (((x - mean) * inv) * weight[i] + (bias ? bias[i] : 0.f)) * out_scale;
+    auto finish = [&](int i, float xv) {
+        const float y = (((xv - mean) * inv) * weight[i] + (bias ? bias[i] : 0.f)) * out_scale;
         if (acc != nullptr) {
             const float sumh = acc[src * width + i] + y;
             acc[src * width + i] = sumh;
@@ -587,6 +607,15 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const elem_t* __restrict
         } else {
             out[(size_t)r * width + i] = from_float<elem_t>(y);
         }
+    };
+    if (kept) {
+#pragma unroll
+        for (int j = 0; j < LN_REGS; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            if (i < width) finish(i, x[j]);
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) finish(i, re ? to_float(re[i]) : rf[i]);
     }
 }
 

@@ -10,8 +10,8 @@
 // it, so a row's result does not depend on the batch.  Accumulation is 32-bit; the bfloat16 engine multiplies on
 // the matrix cores (v_mfma_f32_16x16x32_bf16, operands staged through LDS), the float engine with plain FMAs.
 //
-// Routing (32-bit): `router_topk_kernel` (logits of one token against every expert, sigmoid, the best groups
-// of neighbouring experts, the best experts within them), `route_sort_kernel` (the chosen (token, expert) pairs
+// Routing (32-bit): `router_topk_kernel` (sigmoid of a token's router logits, the best groups of neighbouring
+// experts, the best experts within them), `route_sort_kernel` (the chosen (token, expert) pairs
 // sorted by expert: offsets, the token of every sorted row, the sorted row of every pair),
 // `route_combine_kernel` (a token's output: the weighted sum of its experts' rows, in the order of its choices).
 #include "common.h"
@@ -119,8 +119,9 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GroupedArgs g) {
 #else
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
-#define GBK 32
-#define GLDS (GBK + 8)           // elements between staged rows: 80 bytes
+#define GBK 128
+#define GLDS (GBK + 8)           // elements between staged rows: 272 bytes, so that 16 rows' 16-byte reads meet no bank twice
+#define GCHUNKS (GBK / 8 / 4)    // 16-byte chunks of a row that one thread stages (four threads a row)
 
 __device__ __forceinline__ bf16x8 load_k8(const __bf16* p, int k, int K, bool vector_ok) {
     bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -134,10 +135,11 @@ __device__ __forceinline__ bf16x8 load_k8(const __bf16* p, int k, int K, bool ve
     return v;
 }
 
-// Workgroup tile 64 x 64: 2 x 2 wavefronts of 2 x 2 tiles of 16 x 16.
+// Workgroup tile 64 x 64: 2 x 2 wavefronts of 2 x 2 tiles of 16 x 16; blocks of 128 k staged through LDS, the next
+// block on its way from memory into registers meanwhile (a block's loads are all asked for before anything waits).
 __global__ __launch_bounds__(256) void grouped_gemm_kernel(GroupedArgs g) {
-    __shared__ __bf16 as[GBM * GLDS];
-    __shared__ __bf16 ws[GBN * GLDS];
+    __shared__ __attribute__((aligned(16))) __bf16 as[GBM * GLDS];
+    __shared__ __attribute__((aligned(16))) __bf16 ws[GBN * GLDS];
     int group, m0, m_end;
     tile_of(g, group, m0, m_end);
     if (group < 0 || m0 >= m_end) return;
@@ -150,35 +152,52 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GroupedArgs g) {
     const bool a_vec = (g.K % 8) == 0 && (g.lda % 8) == 0 && (g.a_group % 8) == 0 &&
                        (reinterpret_cast<uintptr_t>(g.a) % 16) == 0;
     const bool w_vec = (g.K % 8) == 0 && (g.w_group % 8) == 0 && (reinterpret_cast<uintptr_t>(g.w) % 16) == 0;
-    const int srow = t >> 2, skc = (t & 3) * 8;      // this thread stages 8 k of row srow of both operands
+    const int srow = t >> 2, sk = (t & 3) * 8;       // this thread stages row srow of both operands: chunks sk + 32 c
     long arow = -1;
     if (m0 + srow < m_end) arow = g.gather ? g.gather[m0 + srow] : m0 + srow;
     const bool wrow_ok = n0 + srow < g.N;
+    const __bf16* ap = a + (arow >= 0 ? arow : 0) * g.lda;
+    const __bf16* wp = w + (size_t)(wrow_ok ? n0 + srow : 0) * g.K;
     floatx4 acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    bf16x8 ar[GCHUNKS], wr[GCHUNKS];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < GCHUNKS; ++c) {
+            const int k = k0 + sk + 32 * c;
+            ar[c] = load_k8(ap, k, g.K, a_vec);
+            wr[c] = load_k8(wp, k, g.K, w_vec);
+        }
+    };
+    fetch(0);
     for (int k0 = 0; k0 < g.K; k0 += GBK) {
-        *reinterpret_cast<bf16x8*>(&as[srow * GLDS + skc]) =
-            arow >= 0 ? load_k8(a + arow * g.lda, k0 + skc, g.K, a_vec) : zero;
-        *reinterpret_cast<bf16x8*>(&ws[srow * GLDS + skc]) =
-            wrow_ok ? load_k8(w + (size_t)(n0 + srow) * g.K, k0 + skc, g.K, w_vec) : zero;
+#pragma unroll
+        for (int c = 0; c < GCHUNKS; ++c) {
+            *reinterpret_cast<bf16x8*>(&as[srow * GLDS + sk + 32 * c]) = arow >= 0 ? ar[c] : zero;
+            *reinterpret_cast<bf16x8*>(&ws[srow * GLDS + sk + 32 * c]) = wrow_ok ? wr[c] : zero;
+        }
         __syncthreads();
-        bf16x8 af[2], wf[2];
+        if (k0 + GBK < g.K) fetch(k0 + GBK);
         const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-            af[i] = *reinterpret_cast<const bf16x8*>(&as[((wm * 2 + i) * 16 + frag_row) * GLDS + frag_k]);
+        for (int kk = 0; kk < GBK; kk += 32) {
+            bf16x8 af[2], wf[2];
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-            wf[j] = *reinterpret_cast<const bf16x8*>(&ws[((wn * 2 + j) * 16 + frag_row) * GLDS + frag_k]);
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 2; ++i)
+                af[i] = *reinterpret_cast<const bf16x8*>(&as[((wm * 2 + i) * 16 + frag_row) * GLDS + kk + frag_k]);
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+                wf[j] = *reinterpret_cast<const bf16x8*>(&ws[((wn * 2 + j) * 16 + frag_row) * GLDS + kk + frag_k]);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+        }
         __syncthreads();
     }
     // accumulator element r of a lane: row (lane / 16) * 4 + r, column lane % 16
@@ -219,35 +238,18 @@ __device__ __forceinline__ void wave_best(float& value, int& index) {
     }
 }
 
-// One wavefront a token.  z[e] = x . router[e] (32-bit sums), s = sigmoid(z).  The experts form `group_count`
+// One wavefront a token.  s = sigmoid(z), z[m] the token's router logits (float: a product of the framework's own,
+// 32-bit sums).  The experts form `group_count`
 // equal groups of neighbours; a group's score is the sum of its two largest s (of its only one, when a group is
 // one expert); only experts of the `group_keep` best groups stand; of those the `top` largest s are chosen
 // (ties: the lower index), ids[m][i] in descending order of s with weights[m][i] = s itself.
-__global__ __launch_bounds__(64) void router_topk_kernel(const elem_t* __restrict__ x, long ldx,
-                                                         const float* __restrict__ router, int32_t* __restrict__ ids,
-                                                         float* __restrict__ weights, int width, int experts, int top,
+__global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict__ z, int32_t* __restrict__ ids,
+                                                         float* __restrict__ weights, int experts, int top,
                                                          int group_count, int group_keep) {
     __shared__ float s_lds[MAX_EXPERTS];
     __shared__ float g_lds[MAX_EXPERTS];
     const int m = blockIdx.x, lane = threadIdx.x;
-    const elem_t* row = x + (size_t)m * ldx;
-    // eight experts a pass over the row: a lane's sum for an expert takes the row's elements in ascending order
-    for (int e0 = 0; e0 < experts; e0 += 8) {
-        float part[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) part[j] = 0.f;
-        for (int i = lane; i < width; i += 64) {
-            const float xv = to_float(row[i]);
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                if (e0 + j < experts) part[j] = fmaf(xv, router[(size_t)(e0 + j) * width + i], part[j]);
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float z = wave_sum(part[j]);
-            if (lane == 0 && e0 + j < experts) s_lds[e0 + j] = 1.0f / (1.0f + expf(-z));
-        }
-    }
+    for (int e = lane; e < experts; e += 64) s_lds[e] = 1.0f / (1.0f + expf(-z[(size_t)m * experts + e]));
     __syncthreads();
     const int per = experts / group_count;
     for (int gidx = lane; gidx < group_count; gidx += 64) {
@@ -374,14 +376,13 @@ int mlr_grouped_gemm(const void* a, long lda, long a_group, const void* w, long 
     return (int)hipGetLastError();
 }
 
-int mlr_router_topk(const void* x, long ldx, const float* router, int32_t* ids, float* weights, int rows, int width,
-                    int experts, int top, int group_count, int group_keep, hipStream_t stream) {
+int mlr_router_topk(const float* z, int32_t* ids, float* weights, int rows, int experts, int top, int group_count,
+                    int group_keep, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (experts < 1 || experts > MAX_EXPERTS || group_count < 1 || experts % group_count != 0 || group_keep < 1 ||
         group_keep > group_count || top < 1 || top > group_keep * (experts / group_count))
         return -1;
-    router_topk_kernel<<<rows, 64, 0, stream>>>((const elem_t*)x, ldx, router, ids, weights, width, experts, top,
-                                                group_count, group_keep);
+    router_topk_kernel<<<rows, 64, 0, stream>>>(z, ids, weights, experts, top, group_count, group_keep);
     return (int)hipGetLastError();
 }
 

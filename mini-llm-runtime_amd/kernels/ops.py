@@ -1244,16 +1244,13 @@ class Kernels:
             ctypes.c_long(0), _p(offsets), _p(gather), _c_int(rows), _c_int(n), _c_int(k), _c_int(experts),
             _c_int(self.GROUPED_ACTS[act]), _c_int(0), _stream()), "experts_gemm")
 
-    @timed("gemm")
-    def router_topk(self, x, router, ids, weights, group_count, group_keep):
-        """Per row of x [rows, width]: s = sigmoid(x . router^T) (router float [experts, width], sums 32-bit); of the
-        group_count equal groups of neighbouring experts the group_keep with the largest sum of their two best s stay;
-        ids [rows, top] int32 the experts with the largest s among those, weights [rows, top] float their s."""
-        _tensor(x, "x", self.dtype, ndim=2)
-        rows, width = x.shape
-        _tensor(router, "router", torch.float32, ndim=2)
-        experts = router.shape[0]
-        _need(router.shape[1] == width, "router: wrong width")
+    @timed("activation", _tensors_work())
+    def router_topk(self, logits, ids, weights, group_count, group_keep):
+        """Per row of the router logits [rows, experts] (float): s = sigmoid(z); of the group_count equal groups of
+        neighbouring experts the group_keep with the largest sum of their two best s stay; ids [rows, top] int32 the
+        experts with the largest s among those, weights [rows, top] float their s."""
+        _tensor(logits, "logits", torch.float32, ndim=2)
+        rows, experts = logits.shape
         _tensor(ids, "ids", torch.int32, ndim=2)
         top = ids.shape[1]
         _need(ids.shape[0] == rows, "ids: one row a token")
@@ -1261,9 +1258,9 @@ class Kernels:
         _need(1 <= experts <= self.MAX_EXPERTS and group_count >= 1 and experts % group_count == 0
               and 1 <= group_keep <= group_count and 1 <= top <= group_keep * (experts // group_count),
               "router_topk: experts up to 256 in equal groups, and no more choices than the kept groups hold")
-        _ok(self._lib("grouped_gemm").mlr_router_topk(_p(x), ctypes.c_long(width), _p(router), _p(ids), _p(weights),
-                                                      _c_int(rows), _c_int(width), _c_int(experts), _c_int(top),
-                                                      _c_int(group_count), _c_int(group_keep), _stream()), "router_topk")
+        _ok(self._lib("grouped_gemm").mlr_router_topk(_p(logits), _p(ids), _p(weights), _c_int(rows), _c_int(experts),
+                                                      _c_int(top), _c_int(group_count), _c_int(group_keep), _stream()),
+            "router_topk")
 
     @timed("gemm")
     def route_sort(self, ids, experts, offsets, token_of, row_of):

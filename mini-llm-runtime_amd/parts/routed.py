@@ -1,5 +1,5 @@
 """A mixture of experts with group-limited routing.  Every token scores all experts, s = sigmoid(router . x) in
-32-bit; the experts form equal groups of neighbours, a group's score is the sum of its two largest s, and only
+32-bit (an ordinary product with float output); the experts form equal groups of neighbours, a group's score is the sum of its two largest s, and only
 experts of the best groups can be chosen; of those the `top` largest s win and weigh their experts' outputs (as
 they are, or divided by their sum).  An expert is an ungated feed-forward down(act(up(x))).
 
@@ -33,7 +33,9 @@ class RoutedMlp:
 
     def weight_specs(self):
         s = self.spec
-        specs = {"router": WeightSpec((s.experts, s.hidden), keep_float32=True, init=("normal", 0.0, 0.05))}
+        # (a matrix like the others: its products with the layer's input are exact in 32 bits, and so are their sums'
+        # partial results up to rounding: the logits are an ordinary product with float output)
+        specs = {"router": WeightSpec((s.experts, s.hidden), init=("normal", 0.0, 0.05))}
         for e in range(s.experts):
             specs[f"e{e}.up"] = WeightSpec((s.intermediate, s.hidden), stack="up")
         for e in range(s.experts):
@@ -47,12 +49,13 @@ class RoutedMlp:
         self.down = stacked([weights[f"e{e}.down"] for e in range(s.experts)]).view(s.experts, s.hidden, s.intermediate)
 
     def libraries(self):
-        return ["grouped_gemm"]
+        return ["gemm", "grouped_gemm"]
 
     def workspace_plan(self, rows, dtype, limits):
         s = self.spec
         pairs = rows * s.top
-        return {("route_ids", torch.int32): pairs, ("route_weights", torch.float32): pairs,
+        return {("route_logits", torch.float32): rows * s.experts, ("route_ids", torch.int32): pairs,
+                ("route_weights", torch.float32): pairs,
                 ("route_offsets", torch.int32): s.experts + 1, ("route_token", torch.int32): pairs,
                 ("route_row", torch.int32): pairs, ("route_act", dtype): pairs * s.intermediate,
                 ("route_y", dtype): pairs * s.hidden, ("ffn_out", dtype): rows * s.hidden}
@@ -67,7 +70,9 @@ class RoutedMlp:
         offsets = ws.get("route_offsets", (s.experts + 1,), torch.int32)
         token_of = ws.get("route_token", (pairs,), torch.int32)
         row_of = ws.get("route_row", (pairs,), torch.int32)
-        k.router_topk(x, self.router, ids, weights, s.group_count, s.group_keep)
+        logits = ws.get("route_logits", (m, s.experts), torch.float32)
+        k.gemm(x, self.router, logits)                   # 32-bit sums of the engine's element type's products
+        k.router_topk(logits, ids, weights, s.group_count, s.group_keep)
         k.route_sort(ids, s.experts, offsets, token_of, row_of)
         act = ws.get("route_act", (pairs, s.intermediate), x.dtype)
         k.experts_gemm(x, self.up, act, offsets, gather=token_of, act=s.activation)

@@ -395,9 +395,13 @@ def test_router_against_the_plain_choice(dtype_name, experts, top, count, keep):
     router = (rng.normal(size=(experts, width)) * 0.4).astype(np.float32).astype(np.float64)
     cfg = dict(experts=experts, top=top, groups=dict(count=count, keep=keep))
     chosen, weights = P.route(x, {"router": router}, cfg)
+    router = as_rounded(router, dtype)
+    chosen, weights = P.route(x, {"router": router}, cfg)
     ids = torch.empty((m, top), dtype=torch.int32, device="cuda")
     wts = torch.empty((m, top), dtype=torch.float32, device="cuda")
-    k.router_topk(on_gpu(x, dtype), on_gpu(router, torch.float32), ids, wts, count, keep)
+    logits = torch.empty((m, experts), dtype=torch.float32, device="cuda")
+    k.gemm(on_gpu(x, dtype), on_gpu(router, dtype), logits)
+    k.router_topk(logits, ids, wts, count, keep)
     got_ids, got_w = ids.cpu().numpy(), wts.double().cpu().numpy()
     s = 1 / (1 + np.exp(-(x @ router.T)))
     for r in range(m):
