@@ -52,8 +52,8 @@ CONFIGS = {
     "wide_view": model(64, 64, [dense(latent(8, 8, 8, 8, 16, 1000), 96), dense(chunked(8, 8, 8, 8, 4, 1000), 96)]),
     "edges": model(160, 80, [dense(latent(5, 16, 16, 16, 32, 100), 96), dense(chunked(4, 1, 16, 32, 8, 128), 96),
                              dense(latent(2, 32, 8, 48, 64, 333), None)]),
-    "matrix_sizes": model(128, 128, [moe(latent(4, 32, 32, 32, 96, 64), 64, 8, 2, 2, 1), dense(chunked(8, 2, 64, 64, 32, 64), 256)],
-                          logit_scale=0.25),
+    "matrix_sizes": model(128, 128, [moe(latent(4, 32, 32, 32, 64, 72), 64, 12, 3, 3, 2), dense(chunked(8, 2, 64, 48, 32, 80), 256)],
+                          logit_scale=0.75),
 }
 LENGTHS = [70, 33, 150, 17, 64, 129, 2, 45]
 _cache = {}
@@ -219,7 +219,7 @@ def groups_of(count_rows, size):
 
 @pytest.mark.parametrize("kind,size", [("window", 37), ("chunk", 24), ("window", 1), ("chunk", 1), ("all", 0), ("window", 150), ("chunk", 64)])
 @pytest.mark.parametrize("heads,kv,dim,vdim,shared,page", [(4, 2, 32, 16, False, 8), (3, 1, 24, 80, False, 4), (8, 8, 64, 64, False, 16),
-                                                           (5, 1, 112, 96, True, 16), (16, 1, 200, 160, True, 8), (2, 1, 576, 512, True, 16),
+                                                           (5, 1, 104, 80, True, 16), (16, 1, 200, 160, True, 8), (2, 1, 576, 512, True, 16),
                                                            (96, 1, 40, 32, True, 8)])
 def test_matrix_core_attention_in_groups_of_tokens_and_of_single_tokens(kind, size, heads, kv, dim, vdim, shared, page):
     """Every position of a request of 210 tokens at once, in the workgroups of prompt portions (groups of consecutive
@@ -383,7 +383,7 @@ def test_layer_norm_of_a_sublayers_output_and_of_the_stream(dtype_name, width):
 
 
 @pytest.mark.parametrize("dtype_name", DTYPES)
-@pytest.mark.parametrize("experts,top,count,keep", [(8, 2, 2, 1), (6, 2, 3, 2), (8, 3, 8, 4), (5, 5, 1, 1), (1, 1, 1, 1), (64, 6, 8, 3),
+@pytest.mark.parametrize("experts,top,count,keep", [(8, 2, 4, 1), (6, 2, 3, 2), (8, 3, 8, 4), (5, 5, 1, 1), (1, 1, 1, 1), (64, 6, 8, 3),
                                                      (256, 8, 16, 4), (12, 4, 2, 2)])
 def test_router_against_the_plain_choice(dtype_name, experts, top, count, keep):
     from mini_llm_runtime_amd.kernels import Kernels
