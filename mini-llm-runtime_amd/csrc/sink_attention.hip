@@ -306,6 +306,7 @@ __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, c
     const int m = first + (ti < count ? ti : 0);
     const int qpos = p0 + ti;
     const int qlo = first_seen(qpos, a.mask_kind, a.mask_size);
+    const int last_lo = first_seen(p0 + count - 1, a.mask_kind, a.mask_size);      // (no token's range starts later)
     bf16x8 qf[NKF];
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -328,9 +329,9 @@ __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, c
     // A thread stages the same key of every tile (key = thread % 32: 256 is a multiple of it) and the chunks
     // thread / 32 + 8 i of its row: one row address a tile, then loads that do not wait for each other (addresses
     // are clamped and what must not count is zeroed afterwards: a load behind a branch would wait for the one before).
-    bf16x8 kreg[NSK], vreg[NSV];
+    bf16x8 kreg_a[NSK], vreg_a[NSV];
     const int my_key = tid & 31, my_chunk = tid >> 5;
-    auto fetch = [&](int t0) {
+    auto fetch = [&](int t0, bf16x8 (&kreg)[NSK], bf16x8 (&vreg)[NSV]) {
         const int kp = t0 + my_key;
         const bool inside = kp >= kbegin && kp < kend;
         const int blk = inside ? kp / a.page_size - block0 : 0;
@@ -354,36 +355,43 @@ __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, c
             }
         }
     };
-    auto stage = [&]() {
+    // The transposed values go to LDS two keys a write: neighbouring lanes hold neighbouring keys, so a lane takes its
+    // neighbour's 16-bit halves by a lane exchange (no LDS traffic) and writes the pair (key, key + 1) of a channel as
+    // ONE 32-bit word -- the even lane the even channels, the odd lane the odd ones: half the LDS instructions of
+    // eight 16-bit writes, which were what a tile of wide values waited for.
+    const bool odd_key = my_key & 1;
+    const int key_pair = my_key & ~1;
+    auto transposed = [&](const bf16x8& rows, int d) {
+        typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+        const u32x4 w = __builtin_bit_cast(u32x4, rows);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t own = w[c];
+            const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)own, 0xB1, 0xF, 0xF, true);   // lane ^ 1
+            const uint32_t pair = odd_key ? ((other >> 16) | (own & 0xffff0000u)) : ((own & 0xffffu) | (other << 16));
+            const int channel = d + 2 * c + (odd_key ? 1 : 0);
+            *reinterpret_cast<uint32_t*>(&vt_lds[channel * VT_PITCH + key_pair]) = channel < V ? pair : 0u;
+        }
+    };
+    auto stage = [&](const bf16x8 (&kreg)[NSK], const bf16x8 (&vreg)[NSV]) {
 #pragma unroll
         for (int i = 0; i < NSK; ++i) {
             const int d = (my_chunk + 8 * i) * 8;
             if (d < KD) {
                 *reinterpret_cast<bf16x8*>(&k_lds[my_key * KP + d]) = kreg[i];
-                if (shared_rows && d < NVT * 16) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) vt_lds[(d + e) * VT_PITCH + my_key] = (d + e < V) ? kreg[i][e] : (__bf16)0.f;
-                }
+                if (shared_rows && d < NVT * 16) transposed(kreg[i], d);
             }
         }
         if (!shared_rows) {
 #pragma unroll
             for (int i = 0; i < NSV; ++i) {
                 const int d = (my_chunk + 8 * i) * 8;
-                if (d < NVT * 16) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) vt_lds[(d + e) * VT_PITCH + my_key] = vreg[i][e];
-                }
+                if (d < NVT * 16) transposed(vreg[i], d);
             }
         }
     };
 
-    const int t_first = (kbegin / TK) * TK;
-    fetch(t_first);
-    for (int t0 = t_first; t0 < kend; t0 += TK) {
-        stage();
-        __syncthreads();
-        if (t0 + TK < kend) fetch(t0 + TK);
+    auto tile = [&](int t0) {
         // scores of this lane's column against the tile's keys 8 b .. 8 b + 7
         floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
         const int i16 = lane & 15;
@@ -397,23 +405,26 @@ __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, c
         }
         float sc[8];
         float tile_max = -INFINITY;
+        // a tile that every token of the group sees whole needs no comparisons (the same in every thread)
+        const bool whole = t0 >= last_lo && t0 + TK - 1 <= p0;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const int kp = t0 + 8 * b + e;
             const float raw = e < 4 ? s0[e] : s1[e - 4];
-            const bool seen = col_ok && kp >= qlo && kp <= qpos;
+            const bool seen = col_ok && (whole || (kp >= qlo && kp <= qpos));
             sc[e] = seen ? raw * scale2 : -INFINITY;
             tile_max = fmaxf(tile_max, sc[e]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, MLR_WAVE));
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, MLR_WAVE));
         const float new_max = fmaxf(run_max, tile_max);
-        const float corr = new_max > -INFINITY ? exp2f(run_max - new_max) : 1.f;
+        // (the raw exponential instruction: its arguments are at most 0, and what underflows may be 0)
+        const float corr = new_max > -INFINITY ? __builtin_amdgcn_exp2f(run_max - new_max) : 1.f;
         float part = 0.f;
         bf16x8 pf;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float p = new_max > -INFINITY ? exp2f(sc[e] - new_max) : 0.f;      // (exp2(-inf) = 0 for unseen keys)
+            const float p = new_max > -INFINITY ? __builtin_amdgcn_exp2f(sc[e] - new_max) : 0.f;
             part += p;
             pf[e] = (__bf16)p;
         }
@@ -421,15 +432,28 @@ __global__ __launch_bounds__(256) void sink_attention_tiles_kernel(SinkArgs a, c
         part += __shfl_xor(part, 32, MLR_WAVE);
         run_sum = run_sum * corr + part;
         run_max = new_max;
+        // the sums so far are only scaled where some column's maximum rose (the same in every lane of the wavefront)
+        const bool rose = __builtin_amdgcn_ballot_w64(corr != 1.f) != 0;
 #pragma unroll
         for (int j = 0; j < NACC; ++j) {
             const int vt = SPLITV ? j * 4 + wave : j;
             if (vt * 16 < V) {                     // (the same in every lane)
-                acc[j] *= corr;
+                if (rose) acc[j] *= corr;
                 const bf16x8 av = *reinterpret_cast<const bf16x8*>(&vt_lds[(vt * 16 + i16) * VT_PITCH + 8 * b]);
                 acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pf, acc[j], 0, 0, 0);
             }
         }
+    };
+    // The next tile's rows are asked for before this tile's products, unconditionally (beyond the range the rows come
+    // out as zeros): a load behind a branch would make the loop wait for it where the branches join, before the
+    // products it is meant to hide behind.
+    const int t_first = (kbegin / TK) * TK;
+    fetch(t_first, kreg_a, vreg_a);
+    for (int t0 = t_first; t0 < kend; t0 += TK) {
+        stage(kreg_a, vreg_a);
+        __syncthreads();
+        fetch(t0 + TK, kreg_a, vreg_a);
+        tile(t0);
         __syncthreads();
     }
     if (a.partial != nullptr) {                // this range's share: the merge kernel finishes the column
