@@ -169,11 +169,12 @@ def plain_attend(q, keys, values, positions, kind, size, sink, scale, group):
 
 @pytest.mark.parametrize("dtype_name", DTYPES)
 @pytest.mark.parametrize("kind,size", [("window", 37), ("chunk", 24), ("window", 1), ("chunk", 1), ("all", 0), ("window", 64), ("chunk", 128)])
-@pytest.mark.parametrize("heads,kv,dim,vdim,page", [(4, 2, 32, 16, 8), (3, 1, 20, 70, 4), (2, 2, 80, 24, 16)])
+@pytest.mark.parametrize("heads,kv,dim,vdim,page", [(4, 2, 32, 16, 8), (3, 1, 20, 70, 4), (2, 2, 80, 32, 16)])
 def test_sink_attention_finds_one_key_wherever_it_lies(dtype_name, kind, size, heads, kv, dim, vdim, page):
     """One key among 300 is made to stand out for one query; the query's output must be that key's value when the mask
     lets it through and must not know it when it does not: at the first tokens, at page borders, far back, and just
-    inside and just outside the window or chunk."""
+    inside and just outside the window or chunk.  The scalar kernel, and where it takes the sizes the matrix-core
+    kernel with every query a group of its own (a decoded token), whole and in key ranges."""
     from mini_llm_runtime_amd.kernels import Kernels
     dtype = DTYPES[dtype_name]
     k = Kernels(dtype)
@@ -206,6 +207,21 @@ def test_sink_attention_finds_one_key_wherever_it_lies(dtype_name, kind, size, h
     got = out.double().cpu().numpy()
     assert np.isfinite(got).all()
     np.testing.assert_allclose(got, want, **tolerance(dtype_name))
+    if k.sink_tiles_supported(dim, vdim, dim, vdim, page, None if kind == "all" else kind, size, T):
+        first, count = torch.arange(m, dtype=torch.int32, device="cuda"), torch.ones(m, dtype=torch.int32, device="cuda")
+        big_heads, _, small_heads, small_tokens = k.sink_tiles_layout(heads, kv)
+        for head_block, split, ranges in ((small_heads, True, 0), (big_heads, False, 0), (small_heads, True, 64)):
+            more = {}
+            if ranges:
+                splits = -(-(T + 31) // ranges)
+                more = dict(partial=torch.full((k.sink_partial_numel(m, small_tokens, heads, vdim, splits),), float("nan"), device="cuda"),
+                            split_keys=ranges, splits=splits)
+            out.fill_(float("nan"))
+            k.sink_attention_tiles(on_gpu(q.reshape(m, -1), dtype), k_pages, v_pages, table, torch.zeros(m, dtype=torch.int32, device="cuda"),
+                                   torch.tensor(positions, dtype=torch.int32, device="cuda"), on_gpu(sink, torch.float32), out, first,
+                                   count, m, head_block, split, heads, kv, dim, vdim, page, 1.0, None if kind == "all" else kind, size, T,
+                                   **more)
+            np.testing.assert_allclose(out.double().cpu().numpy(), want, err_msg=str((head_block, split, ranges)), **tolerance(dtype_name))
     seen_pairs = sum(1 for qp, kp in pairs if kind == "all" or (kind == "window" and qp - kp < size) or
                      (kind == "chunk" and qp // size == kp // size))
     assert 0 < seen_pairs and (kind == "all" or seen_pairs < len(pairs))       # both sides of the edge were asked
