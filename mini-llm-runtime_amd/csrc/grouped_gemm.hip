@@ -27,15 +27,15 @@ struct GroupedArgs {
     int M, N, K, groups, act, out_float;
 };
 
-#define GBM 64
+#define GBM 64              // rows and columns of the small workgroup tile (the float engine's only one)
 #define GBN 64
 
 // Which group and which rows this workgroup serves: (group, first row, one beyond the group's last row), or
 // group < 0 when the launch has more workgroups than the groups have tiles.
-__device__ __forceinline__ void tile_of(const GroupedArgs& g, int& group, int& row0, int& row_end) {
+__device__ __forceinline__ void tile_of(const GroupedArgs& g, int& group, int& row0, int& row_end, const int tile_rows = GBM) {
     if (g.offsets == nullptr) {
         group = blockIdx.z;
-        row0 = blockIdx.y * GBM;
+        row0 = blockIdx.y * tile_rows;
         row_end = g.M;
         return;
     }
@@ -43,10 +43,10 @@ __device__ __forceinline__ void tile_of(const GroupedArgs& g, int& group, int& r
     group = -1;
     for (int e = 0; e < g.groups; ++e) {
         const int first = g.offsets[e], count = g.offsets[e + 1] - first;
-        const int tiles = (count + GBM - 1) / GBM;
+        const int tiles = (count + tile_rows - 1) / tile_rows;
         if (tile < tiles) {
             group = e;
-            row0 = first + tile * GBM;
+            row0 = first + tile * tile_rows;
             row_end = first + count;
             return;
         }
@@ -119,10 +119,6 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GroupedArgs g) {
 #else
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
-#define GBK 128
-#define GLDS (GBK + 8)           // elements between staged rows: 272 bytes, so that 16 rows' 16-byte reads meet no bank twice
-#define GCHUNKS (GBK / 8 / 4)    // 16-byte chunks of a row that one thread stages (four threads a row)
-
 __device__ __forceinline__ bf16x8 load_k8(const __bf16* p, int k, int K, bool vector_ok) {
     bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
     if (vector_ok && k + 8 <= K) {
@@ -135,15 +131,22 @@ __device__ __forceinline__ bf16x8 load_k8(const __bf16* p, int k, int K, bool ve
     return v;
 }
 
-// Workgroup tile 64 x 64: 2 x 2 wavefronts of 2 x 2 tiles of 16 x 16; blocks of 128 k staged through LDS, the next
-// block on its way from memory into registers meanwhile (a block's loads are all asked for before anything waits).
+// A workgroup of 2 x 2 wavefronts, each T x T tiles of 16 x 16: T = 2 owns 64 x 64 outputs and takes k in blocks of
+// 128, T = 4 owns 128 x 128 (half the operand traffic an output: for many rows) in blocks of 64.  A block is staged
+// through LDS, the next block on its way from memory into registers meanwhile (a block's loads are all asked for
+// before anything waits).  Rows of a staged block lie 16 bytes further apart than their data, so that the 16-byte
+// reads of 16 rows meet no bank twice.
+template <int T>
 __global__ __launch_bounds__(256) void grouped_gemm_kernel(GroupedArgs g) {
-    __shared__ __attribute__((aligned(16))) __bf16 as[GBM * GLDS];
-    __shared__ __attribute__((aligned(16))) __bf16 ws[GBN * GLDS];
+    constexpr int BM = 32 * T, BN = 32 * T, BK = T == 2 ? 128 : 64, PITCH = BK + 8;
+    constexpr int RT = 256 / BM;                     // threads that share a row of a staged operand
+    constexpr int CH = BK / 8 / RT;                  // 16-byte chunks of it that one thread stages
+    __shared__ __attribute__((aligned(16))) __bf16 as[BM * PITCH];
+    __shared__ __attribute__((aligned(16))) __bf16 ws[BN * PITCH];
     int group, m0, m_end;
-    tile_of(g, group, m0, m_end);
+    tile_of(g, group, m0, m_end, BM);
     if (group < 0 || m0 >= m_end) return;
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, n0 = blockIdx.x * GBN;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, n0 = blockIdx.x * BN;
     const int wm = wave >> 1, wn = wave & 1;
     const __bf16* a = g.a + (g.offsets ? 0 : (size_t)group * g.a_group);
     const __bf16* w = g.w + (size_t)group * g.w_group;
@@ -152,64 +155,64 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GroupedArgs g) {
     const bool a_vec = (g.K % 8) == 0 && (g.lda % 8) == 0 && (g.a_group % 8) == 0 &&
                        (reinterpret_cast<uintptr_t>(g.a) % 16) == 0;
     const bool w_vec = (g.K % 8) == 0 && (g.w_group % 8) == 0 && (reinterpret_cast<uintptr_t>(g.w) % 16) == 0;
-    const int srow = t >> 2, sk = (t & 3) * 8;       // this thread stages row srow of both operands: chunks sk + 32 c
+    const int srow = t / RT, sk = (t % RT) * 8;      // this thread stages row srow of both operands: chunks sk + 8 RT c
     long arow = -1;
     if (m0 + srow < m_end) arow = g.gather ? g.gather[m0 + srow] : m0 + srow;
     const bool wrow_ok = n0 + srow < g.N;
     const __bf16* ap = a + (arow >= 0 ? arow : 0) * g.lda;
     const __bf16* wp = w + (size_t)(wrow_ok ? n0 + srow : 0) * g.K;
-    floatx4 acc[2][2];
+    floatx4 acc[T][T];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < T; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < T; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    bf16x8 ar[GCHUNKS], wr[GCHUNKS];
+    bf16x8 ar[CH], wr[CH];
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int c = 0; c < GCHUNKS; ++c) {
-            const int k = k0 + sk + 32 * c;
+        for (int c = 0; c < CH; ++c) {
+            const int k = k0 + sk + 8 * RT * c;
             ar[c] = load_k8(ap, k, g.K, a_vec);
             wr[c] = load_k8(wp, k, g.K, w_vec);
         }
     };
     fetch(0);
-    for (int k0 = 0; k0 < g.K; k0 += GBK) {
+    for (int k0 = 0; k0 < g.K; k0 += BK) {
 #pragma unroll
-        for (int c = 0; c < GCHUNKS; ++c) {
-            *reinterpret_cast<bf16x8*>(&as[srow * GLDS + sk + 32 * c]) = arow >= 0 ? ar[c] : zero;
-            *reinterpret_cast<bf16x8*>(&ws[srow * GLDS + sk + 32 * c]) = wrow_ok ? wr[c] : zero;
+        for (int c = 0; c < CH; ++c) {
+            *reinterpret_cast<bf16x8*>(&as[srow * PITCH + sk + 8 * RT * c]) = arow >= 0 ? ar[c] : zero;
+            *reinterpret_cast<bf16x8*>(&ws[srow * PITCH + sk + 8 * RT * c]) = wrow_ok ? wr[c] : zero;
         }
         __syncthreads();
-        if (k0 + GBK < g.K) fetch(k0 + GBK);
+        if (k0 + BK < g.K) fetch(k0 + BK);
         const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
 #pragma unroll
-        for (int kk = 0; kk < GBK; kk += 32) {
-            bf16x8 af[2], wf[2];
+        for (int kk = 0; kk < BK; kk += 32) {
+            bf16x8 af[T], wf[T];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                af[i] = *reinterpret_cast<const bf16x8*>(&as[((wm * 2 + i) * 16 + frag_row) * GLDS + kk + frag_k]);
+            for (int i = 0; i < T; ++i)
+                af[i] = *reinterpret_cast<const bf16x8*>(&as[((wm * T + i) * 16 + frag_row) * PITCH + kk + frag_k]);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                wf[j] = *reinterpret_cast<const bf16x8*>(&ws[((wn * 2 + j) * 16 + frag_row) * GLDS + kk + frag_k]);
+            for (int j = 0; j < T; ++j)
+                wf[j] = *reinterpret_cast<const bf16x8*>(&ws[((wn * T + j) * 16 + frag_row) * PITCH + kk + frag_k]);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < T; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < T; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
     }
     // accumulator element r of a lane: row (lane / 16) * 4 + r, column lane % 16
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < T; ++i) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int n = n0 + (wn * 2 + j) * 16 + (lane & 15);
+        for (int j = 0; j < T; ++j) {
+            const int n = n0 + (wn * T + j) * 16 + (lane & 15);
             if (n >= g.N) continue;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int m = m0 + (wm * 2 + i) * 16 + (lane >> 4) * 4 + r;
+                const int m = m0 + (wm * T + i) * 16 + (lane >> 4) * 4 + r;
                 if (m >= m_end) continue;
                 const float y = activate(acc[i][j][r], g.act);
                 const size_t at = out_base + (size_t)m * g.ldo + n;
@@ -369,10 +372,24 @@ int mlr_grouped_gemm(const void* a, long lda, long a_group, const void* w, long 
 #endif
     GroupedArgs g{(const elem_t*)a, lda, a_group, (const elem_t*)w, w_group, out, ldo, out_group, offsets, gather,
                   M, N, K, groups, act, out_float};
+#if MLR_BF16
+    // experts with many rows each: the large tile (310 -> 340 TFLOP/s at 2048 tokens of width 2048, 390 -> 420 at width
+    // 4096; the products a head, with inner sizes of 128 to 512, are faster on the small one)
+    if (offsets != nullptr && (long)M >= 256L * groups && N >= 128) {
+        const int row_tiles = (M + 127) / 128 + (offsets ? groups : 0);
+        if (row_tiles > 65535 || groups > 65535) return -2;
+        grouped_gemm_kernel<4><<<dim3((N + 127) / 128, row_tiles, offsets ? 1 : groups), 256, 0, stream>>>(g);
+        return (int)hipGetLastError();
+    }
+#endif
     const int row_tiles = (M + GBM - 1) / GBM + (offsets ? groups : 0);
     if (row_tiles > 65535 || groups > 65535) return -2;
     dim3 grid((N + GBN - 1) / GBN, row_tiles, offsets ? 1 : groups);
+#if MLR_BF16
+    grouped_gemm_kernel<2><<<grid, 256, 0, stream>>>(g);
+#else
     grouped_gemm_kernel<<<grid, 256, 0, stream>>>(g);
+#endif
     return (int)hipGetLastError();
 }
 
